@@ -17,9 +17,12 @@ from .spec import ModelSpec
 
 
 def inv_frequencies(spec: ModelSpec) -> torch.Tensor:
-    d = spec.head_dim
-    inv = 1.0 / (spec.rope_theta ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
-    rs = spec.rope_scaling
+    return scaled_inv_frequencies(spec.head_dim, spec.rope_theta, spec.rope_scaling)
+
+
+def scaled_inv_frequencies(d: int, theta: float, rs) -> torch.Tensor:
+    """theta^(-2i / d) for i < d / 2 (float64), rescaled as `rs` (a `RopeScaling`, or None) says."""
+    inv = 1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float64) / d))
     if rs is not None and rs.rope_type == "linear":
         inv = inv / rs.factor                      # positions divided by the factor
     elif rs is not None and rs.rope_type == "yarn":
@@ -27,7 +30,7 @@ def inv_frequencies(spec: ModelSpec) -> torch.Tensor:
         # (extrapolated), those that turn fewer than beta_slow times are divided by the factor
         # (interpolated), a linear ramp over the dimension index in between.
         def corr_dim(rotations):
-            return d * math.log(rs.original_max_position_embeddings / (rotations * 2 * math.pi)) / (2 * math.log(spec.rope_theta))
+            return d * math.log(rs.original_max_position_embeddings / (rotations * 2 * math.pi)) / (2 * math.log(theta))
         low, high = corr_dim(rs.beta_fast), corr_dim(rs.beta_slow)
         if rs.truncate:
             low, high = math.floor(low), math.ceil(high)
@@ -53,7 +56,10 @@ def inv_frequencies(spec: ModelSpec) -> torch.Tensor:
 
 def attention_factor(spec: ModelSpec) -> float:
     """What cos and sin are multiplied by (YaRN: 0.1 ln(factor) + 1 unless the config gives it; 1 otherwise)."""
-    rs = spec.rope_scaling
+    return scaling_attention_factor(spec.rope_scaling)
+
+
+def scaling_attention_factor(rs) -> float:
     if rs is None or rs.rope_type != "yarn":
         return 1.0
     if rs.attention_factor is not None:
@@ -67,6 +73,14 @@ def build_rope_table(spec: ModelSpec, max_pos: int, device="cpu"):
     pos = torch.arange(max_pos, dtype=torch.float64)
     ang = torch.outer(pos, inv)
     f = attention_factor(spec)
+    return (ang.cos() * f).float().to(device), (ang.sin() * f).float().to(device)
+
+
+def rope_table(dims: int, theta: float, rs, max_pos: int, device="cpu"):
+    """(cos, sin), each `[max_pos, dims / 2]` fp32, for a mixer that rotates the first `dims` entries of its vectors
+    (angles are formed in float64 and rounded once)."""
+    ang = torch.outer(torch.arange(max_pos, dtype=torch.float64), scaled_inv_frequencies(dims, theta, rs))
+    f = scaling_attention_factor(rs)
     return (ang.cos() * f).float().to(device), (ang.sin() * f).float().to(device)
 
 

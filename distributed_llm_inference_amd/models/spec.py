@@ -64,14 +64,28 @@ class LayerSpec:
     range by a running maximum, over a [dim, vdim] state, a [dim] normaliser and the maximum per head.
     ``parallel``: the mixers in `branches` read the same input; their outputs are RMS-normed over the width
     and averaged.
+    ``rglru``: a real-gated linear recurrent unit over `rec_width` channels: one branch gelu_tanh(W_y h + b), the other
+    W_x h + b behind a causal convolution of `conv` taps (with bias); per block of rec_width / `blocks` channels two
+    gates sigmoid(square matrix . u + b); a = exp(-8 r softplus(lam)); S <- a S + sqrt(1 - a^2) i u; read-out S * y.
+    ``latent_attention``: causal attention whose keys and values are expanded from a cached latent of `kv_rank` numbers
+    per token (RMS-normed) plus one rotated key part of `rot_dim` shared by all heads; queries come through a latent of
+    `q_rank` (RMS-normed) and carry `dim` unrotated + `rot_dim` rotated entries per head.
     Further switches of ``attention``: `bias_rows` > 0 adds a learned bias per (distance bucket, head) to the
     scaled scores (one bucket per distance below bias_rows / 2, logarithmic buckets up to `bias_max`);
     `head_temp` multiplies a head's scaled scores by a learned number; `sink_learned` makes the sink's score a
     learned number per head instead of 0; `head_gate` multiplies a head's output by the sigmoid of one more
-    projection of the mixer's input.
+    projection of the mixer's input. `maps` = 2: differential attention — q and k hold two maps per head, each a
+    softmax attention of its own over the same values; the head's output is a1 - lambda a2 with
+    lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + `diff`, RMS-normed over the value size and scaled by 1 - `diff`.
+    `keep_first`: with a window, the first keep_first tokens of the sequence stay visible. `softcap` > 0: scaled scores
+    become cap tanh(score / cap). `out_gate`: the concatenated heads are multiplied by sigmoid(W_g h), element by element.
+    `rope_dims` > 0: the first rope_dims entries of every q / k vector are rotated by position, frequencies
+    `rope_base`^(-2i / rope_dims), pairs (2i, 2i + 1) when `rope_interleaved` else (i, i + rope_dims / 2), rescaled
+    by `rope_scaling` when given.
     The feed-forward sublayer is `ff_kind`: ``gated_gelu`` (gelu_tanh(gate) * up, biases), ``gelu`` (up, exact
-    GELU, down; no biases) or ``moe`` (`moe` says how tokens are routed to its experts)."""
-    kind: str                       # "attention" | "delta" | "general_delta" | "mlstm" | "parallel"
+    GELU, down; no biases), ``xielu`` (up, a two-sided quadratic / exponential unit with two learned numbers, down) or
+    ``moe`` (`moe` says how tokens are routed to its experts)."""
+    kind: str                       # "attention" | "delta" | "general_delta" | "mlstm" | "parallel" | "rglru" | "latent_attention"
     heads: int
     kv_heads: int
     dim: int
@@ -93,6 +107,20 @@ class LayerSpec:
     branches: tuple = ()
     ff_kind: str = "gated_gelu"
     moe: Optional["MoeSpec"] = None
+    maps: int = 1
+    diff: float = 0.0
+    keep_first: int = 0
+    softcap: float = 0.0
+    out_gate: bool = False
+    rope_dims: int = 0
+    rope_base: float = 10000.0
+    rope_interleaved: bool = False
+    rope_scaling: Optional[RopeScaling] = None
+    q_rank: int = 0
+    kv_rank: int = 0
+    rot_dim: int = 0
+    rec_width: int = 0
+    blocks: int = 1
 
     @property
     def group(self) -> int:
@@ -101,7 +129,7 @@ class LayerSpec:
     @property
     def has_state(self) -> bool:
         """The mixer keeps a per-sequence state in the sequence's slot."""
-        return self.kind in ("delta", "general_delta", "mlstm") or any(b.has_state for b in self.branches)
+        return self.kind in ("delta", "general_delta", "mlstm", "rglru") or any(b.has_state for b in self.branches)
 
     @property
     def has_ff(self) -> bool:
@@ -117,6 +145,15 @@ class LayerSpec:
         return self.kv_heads if self.kind == "attention" else self.heads
 
     def mixer_param_count(self, width: int) -> int:
+        if self.kind == "rglru":
+            w = self.rec_width
+            return 3 * w * width + 2 * w * (w // self.blocks) + w * (self.conv + 6)
+        if self.kind == "latent_attention":
+            return width * (self.q_rank + self.kv_rank + self.rot_dim) + self.q_rank * self.heads * (self.dim + self.rot_dim) \
+                + self.kv_rank * self.heads * (self.dim + self.vdim) + self.heads * self.vdim * width + self.q_rank + self.kv_rank
+        if self.kind == "attention" and self.maps > 1:
+            qn, kn = self.heads * self.maps * self.dim, self.kv_heads * self.maps * self.dim
+            return width * (qn + kn + self.kv_heads * self.vdim + (2 if self.out_gate else 1) * self.heads * self.vdim) + 4 * self.dim
         if self.kind == "parallel":
             return sum(b.mixer_param_count(width) + width for b in self.branches)
         if self.kind == "general_delta":
@@ -133,7 +170,7 @@ class LayerSpec:
     def ff_param_count(self, width: int) -> int:
         if self.moe is not None:
             return self.moe.experts * (3 * width * self.moe.ff + width)
-        if self.ff_kind == "gelu":
+        if self.ff_kind in ("gelu", "xielu"):
             return 2 * width * self.ff
         return 3 * width * self.ff + 2 * self.ff + width if self.ff else 0
 
@@ -158,7 +195,7 @@ class MoeSpec:
 @dataclass(frozen=True)
 class ModelSpec:
     name: str
-    family: str                     # "llama" | "gpt2" | "letarax" | "nufapel"
+    family: str                     # "llama" | "gpt2" | "letarax" | "nufapel" | "tezesun"
     num_layers: int
     hidden_size: int
     num_heads: int
@@ -196,6 +233,13 @@ class ModelSpec:
     loop: tuple = ()
     learned_positions: bool = False          # a learned vector per position is added to the embedding
     logit_softcap: float = 0.0               # > 0: logits <- cap tanh(logits / cap)
+    # `parallel_block`: a layer has ONE plain-weight RMS norm whose output both sublayers read: x += mixer(h) + ff(h).
+    # `layer_scale`: each sublayer's output is multiplied by a learned vector before the sum. `token_shift`: what the
+    # mixer reads is h + (previous token's h - h) * a learned vector (the previous h is per-sequence state of every layer)
+    parallel_block: bool = False
+    layer_scale: bool = False
+    token_shift: bool = False
+    logit_scale: float = 1.0                 # the logits are multiplied by it
 
     @property
     def is_hybrid(self) -> bool:
@@ -205,7 +249,7 @@ class ModelSpec:
     def has_recurrent_state(self) -> bool:
         """Some layer keeps a per-sequence state that lives in the sequence's slot (not in cache blocks): a sequence
         cannot change slots without its state being moved along."""
-        return any(l.has_state for l in self.layer_specs)
+        return self.token_shift or any(l.has_state for l in self.layer_specs)
 
     def layer_runs(self):
         """[(layer, pass)] in the order the layers run; pass is -1 outside the repeated stretch, else the number of the
@@ -388,6 +432,99 @@ class ModelSpec:
             hf_type="nufapel", layer_specs=tuple(layers), norm_kind="dyt", gated_residual=True, loop=lp,
             learned_positions=True, logit_softcap=float(cfg.get("logit_softcap") or 0.0))
 
+    @staticmethod
+    def from_tezesun_config(cfg: Dict[str, Any], name: str = "") -> "ModelSpec":
+        """Tezesun: parallel layers (one RMS norm feeds the mixer and the feed-forward, both outputs scaled by learned
+        vectors and added), the mixer's input blended with the previous token's. ``layers`` lists for each layer its
+        ``type`` — ``rglru`` (mixer: width, blocks, conv), ``attention`` (differential: heads, kv_heads, dim, vdim, diff,
+        scale, softcap, mask.size / mask.keep_first, rot.dims / base / scaling) or ``latent_attention`` (heads, dim,
+        rot_dim, vdim, q_rank, kv_rank, scale, rot) — and its ``mlp`` (``dense`` with ``ff``, or null). A head of its own,
+        logits times ``logit_scale``. Keys a config leaves out switch their mechanism off."""
+        def rope_of(m, interleaved):
+            rot = m.get("rot") or {}
+            if not rot or not int(rot.get("dims", 0)):
+                return dict(rope_dims=0)
+            if int(rot["dims"]) % 2:
+                raise ValueError("rot.dims must be even")
+            sc, scaling = rot.get("scaling"), None
+            if sc:
+                scaling = RopeScaling(factor=float(sc["factor"]), rope_type="yarn", beta_fast=float(sc["fast"]), beta_slow=float(sc["slow"]),
+                                      original_max_position_embeddings=int(sc["original"]))
+            return dict(rope_dims=int(rot["dims"]), rope_base=float(rot["base"]), rope_interleaved=interleaved, rope_scaling=scaling)
+
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m, mlp = l["mixer"], l.get("mlp")
+            if mlp is not None and mlp.get("kind", "dense") != "dense":
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported (dense is)")
+            ffkw = dict(ff=int(mlp["ff"]) if mlp is not None else 0, ff_kind="xielu")
+            if l["type"] == "rglru":
+                w, nb = int(m["width"]), int(m["blocks"])
+                if w % nb:
+                    raise ValueError(f"layer {i}: {w} channels in {nb} blocks")
+                layers.append(LayerSpec("rglru", heads=nb, kv_heads=nb, dim=w // nb, vdim=w // nb, rec_width=w, blocks=nb,
+                                        conv=int(m["conv"]), **ffkw))
+            elif l["type"] == "attention":
+                if int(m["heads"]) % int(m["kv_heads"]):
+                    raise ValueError(f"layer {i}: {m['heads']} heads over {m['kv_heads']} key / value heads")
+                mask = m.get("mask") or {}
+                win = mask.get("size")
+                layers.append(LayerSpec("attention", heads=int(m["heads"]), kv_heads=int(m["kv_heads"]), dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                        window=int(win) if win else None, keep_first=int(mask.get("keep_first") or 0) if win else 0,
+                                        scale=float(m["scale"]), softcap=float(m.get("softcap") or 0.0), maps=2, diff=float(m["diff"]),
+                                        out_gate=True, **rope_of(m, True), **ffkw))
+            elif l["type"] == "latent_attention":
+                rp = rope_of(m, False)
+                if rp["rope_dims"] > int(m["rot_dim"]):
+                    raise ValueError(f"layer {i}: {rp['rope_dims']} rotated entries in a part of {m['rot_dim']}")
+                layers.append(LayerSpec("latent_attention", heads=int(m["heads"]), kv_heads=1, dim=int(m["dim"]), vdim=int(m["vdim"]),
+                                        scale=float(m["scale"]), q_rank=int(m["q_rank"]), kv_rank=int(m["kv_rank"]), rot_dim=int(m["rot_dim"]),
+                                        **rp, **ffkw))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+        if not layers:
+            raise ValueError("a model needs at least one layer")
+        att = [l for l in layers if l.kind != "rglru"] or layers
+        return ModelSpec(
+            name=name or "tezesun", family="tezesun", num_layers=len(layers), hidden_size=int(cfg["width"]),
+            num_heads=max(l.heads for l in att), num_kv_heads=max(l.kv_heads for l in att),
+            head_dim=max(max(l.dim, l.vdim) for l in att), intermediate_size=max(l.ff for l in layers),
+            vocab_size=int(cfg["vocab"]), max_position=1 << 30, norm_eps=float(cfg["norm"]["eps"]), tie_embeddings=False,
+            bos_token_id=cfg.get("bos_token_id"), eos_token_id=_scalar_eos(cfg.get("eos_token_id")), hf_type="tezesun",
+            layer_specs=tuple(layers), parallel_block=True, layer_scale=True, token_shift=True,
+            logit_scale=float(cfg.get("logit_scale", 1.0)))
+
+    def tezesun_config(self) -> Dict[str, Any]:
+        """The inverse of `from_tezesun_config`."""
+        def rot_of(l):
+            if not l.rope_dims:
+                return None
+            r: Dict[str, Any] = {"base": l.rope_base, "dims": l.rope_dims}
+            if l.rope_scaling is not None:
+                rs = l.rope_scaling
+                r["scaling"] = {"factor": rs.factor, "fast": rs.beta_fast, "slow": rs.beta_slow, "original": rs.original_max_position_embeddings}
+            return r
+
+        out = []
+        for l in self.layer_specs:
+            if l.kind == "rglru":
+                m: Dict[str, Any] = {"width": l.rec_width, "blocks": l.blocks, "conv": l.conv}
+            elif l.kind == "attention":
+                m = {"heads": l.heads, "kv_heads": l.kv_heads, "dim": l.dim, "vdim": l.vdim, "scale": l.scale, "diff": l.diff}
+                if l.softcap > 0:
+                    m["softcap"] = l.softcap
+                if l.window:
+                    m["mask"] = {"size": l.window, "keep_first": l.keep_first}
+            else:
+                m = {"heads": l.heads, "dim": l.dim, "rot_dim": l.rot_dim, "vdim": l.vdim, "q_rank": l.q_rank, "kv_rank": l.kv_rank,
+                     "scale": l.scale}
+            if l.kind != "rglru" and rot_of(l) is not None:
+                m["rot"] = rot_of(l)
+            out.append({"type": l.kind, "mixer": m, "mlp": {"kind": "dense", "ff": l.ff} if l.ff else None})
+        return {"architecture": "Tezesun", "layers": out, "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size,
+                "width": self.hidden_size, "logit_scale": self.logit_scale, "bos_token_id": self.bos_token_id,
+                "eos_token_id": self.eos_token_id}
+
     def nufapel_config(self) -> Dict[str, Any]:
         """The inverse of `from_nufapel_config` (`bias_rows` and `rank` are sizes a checkpoint's tensors give; they are
         written so that random weights of the same shapes can be drawn from the config alone)."""
@@ -437,6 +574,8 @@ class ModelSpec:
             return ModelSpec.from_letarax_config(cfg, name=name)
         if cfg.get("architecture") == "Nufapel":
             return ModelSpec.from_nufapel_config(cfg, name=name)
+        if cfg.get("architecture") == "Tezesun":
+            return ModelSpec.from_tezesun_config(cfg, name=name)
         if mt == "gpt2" or any("GPT2" in a for a in archs):
             if cfg.get("activation_function", "gelu_new") != "gelu_new" or cfg.get("scale_attn_by_inverse_layer_idx"):
                 raise ValueError("GPT-2 variants other than gelu_new MLPs with plain 1/sqrt(d) attention scaling are not supported")
@@ -568,7 +707,7 @@ class ModelSpec:
     def hf_config(self) -> Dict[str, Any]:
         """The inverse of `from_hf_config`: a config.json dict for this spec."""
         if self.is_hybrid:
-            return self.nufapel_config() if self.family == "nufapel" else self.letarax_config()
+            return {"nufapel": self.nufapel_config, "tezesun": self.tezesun_config}.get(self.family, self.letarax_config)()
         if self.is_gpt2:
             return {
                 "model_type": "gpt2", "architectures": ["GPT2LMHeadModel"],
@@ -716,12 +855,41 @@ def nufapel_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
                      gated_residual=True, loop=loop, learned_positions=True, logit_softcap=30.0)
 
 
+def tezesun_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int, ff: int, num_layers: int, window: int = 1024,
+                 vocab_size: int = 32000, pattern: str = "lrra", blocks: int = 0, conv: int = 4, q_rank: int = 0, kv_rank: int = 0,
+                 rot_dim: int = 0, keep_first: int = 4) -> ModelSpec:
+    """A Tezesun stack from a few numbers: `pattern` repeats over the layers ('r' recurrent unit over `width` channels, 'a'
+    differential attention whose two maps have head_dim / 2 entries each and whose values have head_dim, window + kept
+    first tokens, rescaled interleaved rotation, 'l' latent attention with head_dim unrotated entries per head), every
+    layer with a feed-forward of `ff`."""
+    rot_dim = rot_dim or max(2, head_dim // 2)
+    rec = LayerSpec("rglru", heads=blocks or heads, kv_heads=blocks or heads, dim=width // (blocks or heads), vdim=width // (blocks or heads),
+                    rec_width=width, blocks=blocks or heads, conv=conv, ff=ff, ff_kind="xielu")
+    dm = max(2, head_dim // 2)
+    att = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=dm, vdim=head_dim, window=window, keep_first=keep_first,
+                    scale=dm ** -0.5, softcap=30.0, maps=2, diff=0.5, out_gate=True, rope_dims=dm, rope_base=500000.0, rope_interleaved=True,
+                    rope_scaling=RopeScaling(factor=8.0, rope_type="yarn", beta_fast=32.0, beta_slow=1.0, original_max_position_embeddings=1024),
+                    ff=ff, ff_kind="xielu")
+    lat = LayerSpec("latent_attention", heads=heads, kv_heads=1, dim=head_dim, vdim=head_dim, scale=(head_dim + rot_dim) ** -0.5,
+                    q_rank=q_rank or max(8, width // 2), kv_rank=kv_rank or max(8, width // 8), rot_dim=rot_dim, rope_dims=rot_dim,
+                    rope_base=250000.0, ff=ff, ff_kind="xielu")
+    kinds = {"r": rec, "a": att, "l": lat}
+    layers = tuple(kinds[pattern[i % len(pattern)]] for i in range(num_layers))
+    return ModelSpec(name=name, family="tezesun", num_layers=num_layers, hidden_size=width, num_heads=heads, num_kv_heads=kv_heads,
+                     head_dim=head_dim, intermediate_size=ff, vocab_size=vocab_size, max_position=1 << 30, norm_eps=1e-5,
+                     tie_embeddings=False, bos_token_id=1, eos_token_id=2, hf_type="tezesun", layer_specs=layers, parallel_block=True,
+                     layer_scale=True, token_shift=True, logit_scale=1.5)
+
+
 # Letarax stacks of the sizes of the Llama benchmark shapes (random weights; `bench.py --hybrid-compare` runs them)
 BUILTIN_SPECS["letarax-1b-like"] = letarax_spec("letarax-1b-like", 2048, 16, 4, 128, 8192, 8, 1024)
 BUILTIN_SPECS["letarax-8b-like"] = letarax_spec("letarax-8b-like", 4096, 32, 8, 128, 14336, 4, 2048)
 # Nufapel stacks of the same sizes (`bench.py --gated-compare` runs them beside the Letarax stacks)
 BUILTIN_SPECS["nufapel-1b-like"] = nufapel_spec("nufapel-1b-like", 2048, 16, 4, 128, 8192, 8)
 BUILTIN_SPECS["nufapel-8b-like"] = nufapel_spec("nufapel-8b-like", 4096, 32, 8, 128, 14336, 4)
+# Tezesun stacks of the same sizes (`bench.py --parallel-compare` runs them beside the Letarax stacks)
+BUILTIN_SPECS["tezesun-1b-like"] = tezesun_spec("tezesun-1b-like", 2048, 16, 4, 128, 8192, 8, window=1024, kv_rank=448, rot_dim=64, q_rank=1024)
+BUILTIN_SPECS["tezesun-8b-like"] = tezesun_spec("tezesun-8b-like", 4096, 32, 8, 128, 14336, 4, window=2048, kv_rank=448, rot_dim=64, q_rank=1536)
 
 
 def _register_test_models():
@@ -741,6 +909,10 @@ def _register_test_models():
                                                       loop=(0, 2, 2), max_position=256, rank=8, bias_rows=8, bias_max=64)
     BUILTIN_SPECS["tiny-nufapel-gpu-test"] = nufapel_spec("tiny-nufapel-gpu-test", 128, 4, 2, 32, 256, 4, vocab_size=320, experts=8,
                                                           loop=(1, 3, 2), max_position=512, rank=16, bias_rows=16, bias_max=200)
+    BUILTIN_SPECS["tiny-tezesun-test"] = tezesun_spec("tiny-tezesun-test", 64, 4, 2, 16, 96, 4, window=12, vocab_size=320, conv=3, blocks=4,
+                                                      q_rank=24, kv_rank=20, rot_dim=8, keep_first=3)
+    BUILTIN_SPECS["tiny-tezesun-gpu-test"] = tezesun_spec("tiny-tezesun-gpu-test", 128, 4, 2, 32, 256, 4, window=40, vocab_size=320, blocks=2,
+                                                          q_rank=48, kv_rank=40, rot_dim=16, keep_first=5)
     BUILTIN_SPECS["tiny-gpt2-gpu-test"] = tiny_spec(
         "gpt2", name="tiny-gpt2-gpu-test", hidden_size=256, num_heads=4, num_kv_heads=4, head_dim=64,
         intermediate_size=1024, vocab_size=333, num_layers=4)

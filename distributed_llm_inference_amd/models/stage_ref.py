@@ -59,6 +59,9 @@ class RefStage:
                 c = [self._fresh_layer_state(self.spec.layer_specs[i]) for i, _ in self.spec.layer_runs()]
             elif self.spec.is_hybrid:
                 c = [self._fresh_layer_state(self.spec.layer_specs[i]) for i in self.plan.layers]
+                if self.spec.token_shift:           # every layer also carries the previous token's normed input
+                    for st in c:
+                        st.append(torch.zeros(self.spec.hidden_size, dtype=torch.float32, device=self.device))
             else:
                 z = lambda: torch.zeros(0, self.spec.num_kv_heads, self.spec.head_dim, dtype=self.dtype, device=self.device)
                 c = [[z(), z()] for _ in self.plan.layers]
@@ -74,8 +77,12 @@ class RefStage:
             return [z32(ls.heads, ls.dim, ls.dim)]
         if ls.kind == "mlstm":
             return [z32(ls.heads, ls.dim, ls.vdim), z32(ls.heads, ls.dim), z32(ls.heads)]
+        if ls.kind == "rglru":
+            return [z32(max(ls.conv - 1, 0), ls.rec_width), z32(ls.rec_width)]
+        if ls.kind == "latent_attention":
+            return [torch.zeros(0, 1, ls.kv_rank, dtype=self.dtype, device=dev), torch.zeros(0, 1, ls.rot_dim, dtype=self.dtype, device=dev)]
         if ls.kind == "attention":
-            return [torch.zeros(0, ls.kv_heads, ls.dim, dtype=self.dtype, device=dev),
+            return [torch.zeros(0, ls.kv_heads * ls.maps, ls.dim, dtype=self.dtype, device=dev),
                     torch.zeros(0, ls.kv_heads, ls.vdim, dtype=self.dtype, device=dev)]
         C = 2 * ls.kv_heads * ls.dim + ls.heads * ls.vdim
         return [torch.zeros(ls.conv - 1, C, dtype=torch.float32, device=dev),
@@ -248,10 +255,110 @@ class RefStage:
             self.layer_outputs.append(h)
         return h
 
+    # -- hybrid stacks with parallel layers: one norm feeds the mixer and the feed-forward -------------------------
+    def _parallel_layers(self, batch: StepBatch, h: torch.Tensor) -> torch.Tensor:
+        """x <- x + ls1 * mixer(shifted(n)) + ls2 * ff(n), n = rms(x) w, for every layer. Norms, rotations, scores, the
+        recurrence with its gates, and the residual sum are fp32 whatever the dtype."""
+        from .rope import rope_table
+        spec, dt, eps, w = self.spec, self.dtype, self.spec.norm_eps, self.w
+        T, dev = h.shape[0], self.device
+        F = torch.nn.functional
+        lin = lambda x, m, b=None: R.gemm(x.to(dt), m, b, None, 1 if b is not None else 0)
+        rnd = lambda x: x.to(dt).float()
+        seqs, t0 = [], 0
+        for slot, qlen, ctx in zip(batch.slots, batch.q_lens, batch.ctx_lens):
+            if qlen > 0 and ctx == 0:
+                self.cache.pop(slot, None)            # a sequence's first tokens: whatever the slot held before is void
+            if qlen > 0:
+                seqs.append((slot, t0, qlen, ctx))
+            t0 += qlen
+        pos = torch.tensor([c + i for c, q in zip(batch.ctx_lens, batch.q_lens) for i in range(q)], dtype=torch.long, device=dev)
+        far = int(pos.max()) + 1 if T else 1
+        self.layer_outputs = []
+        for li, l in enumerate(w.layers):
+            ls = spec.layer_specs[self.plan.layers[li]]
+            n = R.rmsnorm(h, l["ln1_w"], eps)
+            xm = torch.empty_like(n)
+            for slot, s0, qlen, ctx in seqs:
+                st = self._slot_cache(slot)[li]
+                xm[s0:s0 + qlen], st[-1] = R.token_shift(n[s0:s0 + qlen], st[-1], l["shift"])
+            z = lin(xm, l["w_in"], l.get("b_in"))
+            if ls.rope_dims:
+                cos, sin = rope_table(ls.rope_dims, ls.rope_base, ls.rope_scaling, far, dev)
+            if ls.kind == "rglru":
+                W = ls.rec_width
+                y, xb = R.gelu_tanh(z[:, :W]), z[:, W:]
+                mixed = torch.empty(T, W, dtype=torch.float32, device=dev)
+                for slot, s0, qlen, ctx in seqs:
+                    st, sl = self._slot_cache(slot)[li], slice(s0, s0 + qlen)
+                    u, st[0] = R.short_conv(xb[sl], st[0], l["conv_w"])
+                    u = u + l["conv_b"].float()
+                    gr = torch.sigmoid(R.block_linear(u, l["w_ra"], l["b_ra"]))
+                    gi = torch.sigmoid(R.block_linear(u, l["w_ri"], l["b_ri"]))
+                    S, st[1] = R.rglru_scan(u, gr, gi, l["lam"], st[1])
+                    mixed[sl] = S * y[sl]
+            elif ls.kind == "attention":
+                H, G, d, dv, M = ls.heads, ls.kv_heads, ls.dim, ls.vdim, ls.maps
+                qn, kn, vn = H * M * d, G * M * d, G * dv
+                q, k = z[:, :qn].reshape(T, H * M, d), z[:, qn:qn + kn].reshape(T, G * M, d)
+                if ls.rope_dims:
+                    q, k = R.rope_partial(q, cos, sin, pos, ls.rope_interleaved), R.rope_partial(k, cos, sin, pos, ls.rope_interleaved)
+                v, gate = z[:, qn + kn:qn + kn + vn].reshape(T, G, dv), z[:, qn + kn + vn:]
+                lam = torch.exp((l["lq1"].float() * l["lk1"].float()).sum()) - torch.exp((l["lq2"].float() * l["lk2"].float()).sum()) + ls.diff
+                mixed = torch.empty(T, H, dv, dtype=torch.float32, device=dev)
+                for slot, s0, qlen, ctx in seqs:
+                    st, sl = self._slot_cache(slot)[li], slice(s0, s0 + qlen)
+                    assert st[0].shape[0] >= ctx, f"slot {slot}: cache has {st[0].shape[0]} tokens, step says {ctx}"
+                    st[0] = torch.cat([st[0][:ctx], k[sl].to(dt)])
+                    st[1] = torch.cat([st[1][:ctx], v[sl].to(dt)])
+                    maps = []
+                    for mp in range(M):         # map mp of every head: its own queries and keys over the shared values
+                        maps.append(R.attention(q[sl][:, mp::M], st[0][:, mp::M], st[1], ctx, ls.scale, window=ls.window or 0,
+                                                keep_first=ls.keep_first, softcap=ls.softcap))
+                    o = maps[0] - lam * maps[1] if M == 2 else maps[0]
+                    mixed[sl] = R.rmsnorm(o, torch.ones(dv, device=dev), eps) * (1.0 - ls.diff) if M == 2 else o
+                mixed = mixed.reshape(T, H * dv) * torch.sigmoid(gate)
+            else:
+                H, d, dr, dv, Rk = ls.heads, ls.dim, ls.rot_dim, ls.vdim, ls.kv_rank
+                cq = R.rmsnorm(z[:, :ls.q_rank], l["dq_norm"], eps)
+                q = lin(cq, l["w_uq"]).reshape(T, H, d + dr)
+                c = R.rmsnorm(z[:, ls.q_rank:ls.q_rank + Rk], l["dkv_norm"], eps)
+                kr = z[:, ls.q_rank + Rk:].reshape(T, 1, dr)
+                if ls.rope_dims:
+                    kr = R.rope_partial(kr, cos, sin, pos, ls.rope_interleaved)
+                    q = torch.cat([q[..., :d], R.rope_partial(q[..., d:], cos, sin, pos, ls.rope_interleaved)], dim=-1)
+                mixed = torch.empty(T, H, dv, dtype=torch.float32, device=dev)
+                for slot, s0, qlen, ctx in seqs:
+                    st, sl = self._slot_cache(slot)[li], slice(s0, s0 + qlen)
+                    assert st[0].shape[0] >= ctx, f"slot {slot}: cache has {st[0].shape[0]} tokens, step says {ctx}"
+                    st[0] = torch.cat([st[0][:ctx], c[sl].reshape(qlen, 1, Rk).to(dt)])
+                    st[1] = torch.cat([st[1][:ctx], kr[sl].to(dt)])
+                    n_all = st[0].shape[0]
+                    ku = lin(st[0][:, 0], l["w_uk"]).reshape(n_all, H, d)
+                    vv = lin(st[0][:, 0], l["w_uv"]).reshape(n_all, H, dv)
+                    kk = torch.cat([ku, st[1].float().expand(n_all, H, dr)], dim=-1)
+                    mixed[sl] = R.attention(q[sl], kk, vv, ctx, ls.scale)
+                mixed = mixed.reshape(T, H * dv)
+            add = lin(mixed, l["w_o"]) * l["ls1"].float()
+            if ls.ff:
+                act = R.xielu(lin(n, l["w_up"]), l["act"][0], l["act"][1])
+                add = add + lin(rnd(act), l["w_down"]) * l["ls2"].float()
+            h = h + add
+            self.layer_outputs.append(h)
+        return h
+
     def _forward_hybrid(self, batch: StepBatch, x: torch.Tensor) -> torch.Tensor:
         T = batch.num_tokens
         ids = torch.as_tensor(x).to(self.device).long().reshape(-1)
         assert ids.numel() == T, f"expected {T} token ids, got {ids.numel()}"
+        if self.spec.parallel_block:
+            h = self._parallel_layers(batch, self.w.embed[ids].float())
+            self.last_hidden = h
+            rows = self._out_rows(batch)
+            if not rows:
+                return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+            hn = R.rmsnorm(h[rows], self.w.final_norm_w, self.spec.norm_eps)
+            return R.gemm(hn.to(self.dtype), self.w.lm_head).float() * self.spec.logit_scale
         if self.spec.norm_kind == "dyt":
             pos = torch.tensor([c + i for c, q in zip(batch.ctx_lens, batch.q_lens) for i in range(q)], dtype=torch.long, device=self.device)
             h = self.w.embed[ids].float()

@@ -246,11 +246,108 @@ def _random_nufapel_weights(spec: ModelSpec, plan: StagePlan, seed: int, device,
     return w
 
 
+# ---- Tezesun: checkpoint names <-> the logical layout ----------------------------------------------------------------
+# Per layer: ln1_w (the one norm), ls1 / ls2 (layer scales of mixer / feed-forward), shift (token-shift blend);
+#   rglru:            w_in = y | x (one GEMM) with b_in, conv_w [W, taps], conv_b, w_ra / w_ri [blocks, bw, bw] with b_ra / b_ri, lam, w_o
+#   attention:        w_in = q | k | v | g (one GEMM), lq1, lk1, lq2, lk2, w_o
+#   latent_attention: w_in = dq | dkv (one GEMM), dq_norm, dkv_norm, w_uq, w_uk, w_uv, w_o
+#   feed-forward:     w_up, w_down, act (the two numbers of the activation)
+def _tezesun_layer_names(ls, p: str) -> Dict[str, object]:
+    m, f = p + "mix.", p + "mlp."
+    n: Dict[str, object] = {"ln1_w": p + "norm1", "ls1": p + "ls1", "shift": p + "shift", "w_o": m + "o"}
+    if ls.kind == "rglru":
+        n.update({"w_in": (m + "y", m + "x"), "b_in": (m + "y.b", m + "x.b"), "conv_w": m + "conv", "conv_b": m + "conv.b",
+                  "w_ra": m + "ra", "b_ra": m + "ra.b", "w_ri": m + "ri", "b_ri": m + "ri.b", "lam": m + "lam"})
+    elif ls.kind == "attention":
+        n.update({"w_in": (m + "q", m + "k", m + "v", m + "g"), "lq1": m + "lq1", "lk1": m + "lk1", "lq2": m + "lq2", "lk2": m + "lk2"})
+    else:
+        n.update({"w_in": (m + "dq", m + "dkv"), "dq_norm": m + "dq.norm", "dkv_norm": m + "dkv.norm", "w_uq": m + "uq",
+                  "w_uk": m + "uk", "w_uv": m + "uv"})
+    if ls.ff:
+        n.update({"ls2": p + "ls2", "w_up": f + "up", "w_down": f + "down", "act": f + "act"})
+    return n
+
+
+def _tezesun_in_sizes(ls) -> List[int]:
+    if ls.kind == "rglru":
+        return [ls.rec_width, ls.rec_width]
+    if ls.kind == "attention":
+        return [ls.heads * ls.maps * ls.dim, ls.kv_heads * ls.maps * ls.dim, ls.kv_heads * ls.vdim, ls.heads * ls.vdim]
+    return [ls.q_rank, ls.kv_rank + ls.rot_dim]
+
+
+def _load_tezesun_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) -> StageWeights:
+    w = StageWeights(spec, plan)
+    get = lambda name: rd.get(name).to(device=device, dtype=dtype)
+    w.embed, w.lm_head, w.final_norm_w = get("embed"), get("head"), get("final.norm")
+    for i in plan.layers:
+        l = {}
+        for k, names in _tezesun_layer_names(spec.layer_specs[i], f"l{i}.").items():
+            l[k] = torch.cat([get(x) for x in names], dim=0) if isinstance(names, tuple) else get(names)
+        w.layers.append(l)
+    return w
+
+
+def export_tezesun_state_dict(w: StageWeights) -> Dict[str, torch.Tensor]:
+    """Logical -> checkpoint names (tests, `save` of random models)."""
+    spec = w.spec
+    sd = {"embed": w.embed, "head": w.lm_head, "final.norm": w.final_norm_w}
+    for i, l in zip(w.plan.layers, w.layers):
+        ls = spec.layer_specs[i]
+        for k, names in _tezesun_layer_names(ls, f"l{i}.").items():
+            if isinstance(names, tuple):
+                for x, t in zip(names, torch.split(l[k], _tezesun_in_sizes(ls))):
+                    sd[x] = t
+            else:
+                sd[names] = l[k]
+    return {k: v.detach().clone().contiguous() for k, v in sd.items()}
+
+
+def _random_tezesun_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
+    """Random weights with which every mechanism matters: projections at 1 / sqrt(fan-in), biases, gates, layer scales
+    and blends of order one, decays spread over their range."""
+    H, V = spec.hidden_size, spec.vocab_size
+    w = StageWeights(spec, plan)
+    rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
+    one = lambda name, shape, std: torch.ones(shape, device=device, dtype=dtype) + rn(name, shape, std)
+    w.embed, w.lm_head, w.final_norm_w = rn("embed", (V, H), 1.0), rn("head", (V, H), H ** -0.5), one("final.norm", (H,), 0.1)
+    for i in plan.layers:
+        ls, p = spec.layer_specs[i], f"layers.{i}."
+        l: Dict[str, torch.Tensor] = {"ln1_w": one(p + "ln1_w", (H,), 0.1), "ls1": one(p + "ls1", (H,), 0.3) * 0.5,
+                                      "shift": (rn(p + "shift", (H,), 0.25) + 0.5).clamp(0.0, 1.0)}
+        l["w_in"] = rn(p + "w_in", (sum(_tezesun_in_sizes(ls)), H), H ** -0.5)
+        if ls.kind == "rglru":
+            W, nb, bw = ls.rec_width, ls.blocks, ls.rec_width // ls.blocks
+            l["b_in"], l["conv_w"], l["conv_b"] = rn(p + "b_in", (2 * W,), 0.2), rn(p + "conv_w", (W, ls.conv), 0.6), rn(p + "conv_b", (W,), 0.2)
+            l["w_ra"], l["b_ra"] = rn(p + "w_ra", (nb, bw, bw), bw ** -0.5), rn(p + "b_ra", (nb, bw), 0.5)
+            l["w_ri"], l["b_ri"] = rn(p + "w_ri", (nb, bw, bw), bw ** -0.5), rn(p + "b_ri", (nb, bw), 0.5)
+            l["lam"], n_o = rn(p + "lam", (W,), 1.5) - 2.0, W
+        elif ls.kind == "attention":
+            for k in ("lq1", "lk1", "lq2", "lk2"):
+                l[k] = rn(p + k, (ls.dim,), 0.3)
+            n_o = ls.heads * ls.vdim
+        else:
+            l["dq_norm"], l["dkv_norm"] = one(p + "dq_norm", (ls.q_rank,), 0.1), one(p + "dkv_norm", (ls.kv_rank,), 0.1)
+            l["w_uq"] = rn(p + "w_uq", (ls.heads * (ls.dim + ls.rot_dim), ls.q_rank), 2.0 * ls.q_rank ** -0.5)
+            l["w_uk"] = rn(p + "w_uk", (ls.heads * ls.dim, ls.kv_rank), 2.0 * ls.kv_rank ** -0.5)
+            l["w_uv"] = rn(p + "w_uv", (ls.heads * ls.vdim, ls.kv_rank), ls.kv_rank ** -0.5)
+            n_o = ls.heads * ls.vdim
+        l["w_o"] = rn(p + "w_o", (H, n_o), n_o ** -0.5)
+        if ls.ff:
+            l["ls2"] = one(p + "ls2", (H,), 0.3) * 0.5
+            l["w_up"], l["w_down"] = rn(p + "w_up", (ls.ff, H), H ** -0.5), rn(p + "w_down", (H, ls.ff), ls.ff ** -0.5)
+            l["act"] = rn(p + "act", (2,), 0.5)
+        w.layers.append(l)
+    return w
+
+
 def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
     """Random weights of a hybrid stack, scaled so that activations stay of order one through any depth
     (projections at 1 / sqrt(fan-in), embedding at one) and every bias, convolution tap and gate matters."""
     if spec.family == "nufapel":
         return _random_nufapel_weights(spec, plan, seed, device, dtype)
+    if spec.family == "tezesun":
+        return _random_tezesun_weights(spec, plan, seed, device, dtype)
     H, V = spec.hidden_size, spec.vocab_size
     w = StageWeights(spec, plan)
     rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
@@ -286,6 +383,8 @@ def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, 
 def _load_hybrid_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) -> StageWeights:
     if spec.family == "nufapel":
         return _load_nufapel_weights(rd, spec, plan, device, dtype)
+    if spec.family == "tezesun":
+        return _load_tezesun_weights(rd, spec, plan, device, dtype)
     w = StageWeights(spec, plan)
     get = lambda name: rd.get(name).to(device=device, dtype=dtype)
     if plan.has_embed or plan.has_head:

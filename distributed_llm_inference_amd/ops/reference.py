@@ -48,13 +48,15 @@ def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch
 
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, scale: float,
-              window: int = 0, sink: bool = False, k_pos0: int = 0, temp=None, dist_bias=None, sink_logit=None) -> torch.Tensor:
+              window: int = 0, sink: bool = False, k_pos0: int = 0, temp=None, dist_bias=None, sink_logit=None,
+              keep_first: int = 0, softcap: float = 0.0) -> torch.Tensor:
     """One sequence. q [Tq, Hq, D] are the tokens at absolute positions q_pos0.., k [Tk, Hkv, D] and
     v [Tk, Hkv, Dv] hold positions k_pos0..k_pos0+Tk-1 (reaching at least the last query). Causal, GQA.
     `window` > 0: a query at i sees the keys j with 0 <= i - j < window. `sink`: the softmax's
     denominator has one more term, exp(0), that carries no value (`sink_logit` [Hq]: exp(sink_logit) instead).
     `temp` [Hq] multiplies a head's scaled scores; `dist_bias` [distances, Hq] is added to the scaled score of a
-    key at distance i - j (after `temp`). Returns [Tq, Hq, Dv] fp32."""
+    key at distance i - j (after `temp`). `keep_first`: with a window, the keys at positions below it stay visible.
+    `softcap` > 0: scaled scores become cap tanh(score / cap). Returns [Tq, Hq, Dv] fp32."""
     Tq, Hq, D = q.shape
     Tk, Hkv, _ = k.shape
     g = Hq // Hkv
@@ -63,13 +65,15 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, sc
     s = torch.einsum("qhd,khd->hqk", q.float(), kf) * scale
     qpos = torch.arange(Tq, device=q.device).view(-1, 1) + q_pos0
     kpos = torch.arange(Tk, device=q.device).view(1, -1) + k_pos0
+    if softcap > 0:
+        s = softcap * torch.tanh(s / softcap)
     if temp is not None:
         s = s * temp.float().view(Hq, 1, 1)
     if dist_bias is not None:
         s = s + dist_bias.float()[(qpos - kpos).clamp(min=0)].permute(2, 0, 1)
     hidden = kpos > qpos
     if window and window > 0:
-        hidden = hidden | (qpos - kpos >= window)
+        hidden = hidden | ((qpos - kpos >= window) & (kpos >= keep_first))
     s = s.masked_fill(hidden.unsqueeze(0), float("-inf"))
     if sink:
         last = s.new_zeros(Hq, Tq, 1) if sink_logit is None else sink_logit.float().view(Hq, 1, 1).expand(Hq, Tq, 1)
@@ -176,3 +180,56 @@ def moe_route(scores: torch.Tensor, top: int, groups: int, keep: int, scale: flo
     idx = torch.argsort(masked, dim=-1, descending=True, stable=True)[:, :top]
     val = sf.gather(1, idx)
     return idx, val / (val.sum(-1, keepdim=True) + 1e-20) * scale
+
+
+def xielu(z: torch.Tensor, p, q) -> torch.Tensor:
+    """z > 0: softplus(p) z^2 + z / 2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z / 2."""
+    zf = z.float()
+    ap, aq = F.softplus(torch.as_tensor(p).float()), 0.5 + F.softplus(torch.as_tensor(q).float())
+    return torch.where(zf > 0, ap * zf * zf + 0.5 * zf, aq * (torch.expm1(zf.clamp(max=0.0)) - zf) + 0.5 * zf)
+
+
+def token_shift(h: torch.Tensor, prev: torch.Tensor, mu: torch.Tensor):
+    """h [T, W] consecutive tokens of one sequence, prev [W] the h of the token before them (zeros at the start).
+    Returns (h + (previous h - h) * mu, the last token's h)."""
+    hf = h.float()
+    before = torch.cat([prev.float().unsqueeze(0), hf[:-1]])
+    return hf + (before - hf) * mu.float(), hf[-1]
+
+
+def rope_partial(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch.Tensor, interleaved: bool) -> torch.Tensor:
+    """x [T, heads, D]: the first 2 * cos.shape[1] entries of every vector are rotated by the token's position, pairs
+    (2i, 2i + 1) when `interleaved`, else (i, i + dims / 2); the rest pass. fp32."""
+    half = cos.shape[1]
+    xf = x.float()
+    head, tail = xf[..., :2 * half], xf[..., 2 * half:]
+    c, s = cos[positions.long()].unsqueeze(1).float(), sin[positions.long()].unsqueeze(1).float()
+    if interleaved:
+        u, v = head[..., 0::2], head[..., 1::2]
+        out = torch.stack([u * c - v * s, v * c + u * s], dim=-1).reshape(head.shape)
+    else:
+        u, v = head[..., :half], head[..., half:]
+        out = torch.cat([u * c - v * s, v * c + u * s], dim=-1)
+    return torch.cat([out, tail], dim=-1)
+
+
+def block_linear(x: torch.Tensor, w: torch.Tensor, b=None) -> torch.Tensor:
+    """x [T, blocks * n_in] through one matrix per block: w [blocks, n_out, n_in] (+ b [blocks, n_out]) -> [T, blocks * n_out], fp32."""
+    nb, no, ni = w.shape
+    y = torch.einsum("tbi,boi->tbo", x.float().reshape(-1, nb, ni), w.float())
+    if b is not None:
+        y = y + b.float()
+    return y.reshape(-1, nb * no)
+
+
+def rglru_scan(u: torch.Tensor, r: torch.Tensor, i: torch.Tensor, lam: torch.Tensor, S: torch.Tensor, c: float = 8.0):
+    """Per channel: a = exp(-c r softplus(lam)); S <- a S + sqrt(1 - a^2) i u. u, r, i [T, W], lam, S [W] fp32.
+    Returns (the state after every token [T, W], the last state)."""
+    a = torch.exp(-c * r.float() * F.softplus(lam.float()))
+    x = torch.sqrt(1.0 - a * a) * i.float() * u.float()
+    S = S.float().clone()
+    out = torch.empty_like(x)
+    for t in range(x.shape[0]):
+        S = a[t] * S + x[t]
+        out[t] = S
+    return out, S
