@@ -26,6 +26,19 @@ Stacks with dynamic-tanh pre-norms and gated residuals (`spec.norm_kind == "dyt"
              -> [ up GEMM -> gelu -> down GEMM | router -> plan -> the experts' GEMMs over sorted rows -> weighted sum ]
              -> gated residual add + the next norm
 
+Stacks with parallel layers (`spec.parallel_block`: one RMS norm feeds the mixer and the feed-forward, whose outputs are
+scaled by learned vectors and added together) run through `_layers_par`: per layer
+
+    n = rms(h) w (fp32 and the GEMMs' type)  -> token shift (blend with the previous token's n; the last n is the slot's state)
+             -> ONE input GEMM (all projections of the mixer)
+             -> [ causal conv -> block-diagonal gate GEMM -> gated linear recurrence * gelu(y)
+                | rotation + cache write -> attention over two score maps per head, combined, normed, gated
+                | latent norms -> query up-projection -> rotation + cache write of (latent | rotated key part)
+                  -> per-head absorption of the key up-projection into the query -> attention over the latent rows
+                  -> per-head value up-projection ]
+             -> o GEMM;   up GEMM -> xIELU -> down GEMM (reads n itself)
+             -> h += ls1 * mixer + ls2 * ff, the slot's carried n saved, and the next layer's n (one kernel)
+
 Matrix products take bf16 operands (or fp32: `dtype="fp32"`, everything in true 32-bit) and accumulate in
 fp32; norms, scores, softmax, value mixing, gates, decays and states are fp32 in both modes.
 """
@@ -88,8 +101,12 @@ class HybridGpuStage(GpuStage):
         for i, ls in zip(plan.layers, self.specs):
             if max(ls.dim, ls.vdim) > 512:
                 raise ValueError(f"layer {i}: head sizes up to 512 are supported")
-            if ls.kind == "delta" and not 1 <= ls.conv <= 16:
+            if ls.kind in ("delta", "rglru") and not 1 <= ls.conv <= 16:
                 raise ValueError(f"layer {i}: 1 to 16 convolution taps are supported")
+            if ls.kind == "latent_attention" and (ls.kv_rank + ls.rot_dim > 1024 or ls.kv_rank > 512):
+                raise ValueError(f"layer {i}: latents up to 512 (with the rotated part up to 1024) are supported")
+            if ls.kind == "attention" and ls.maps * ls.dim > 1024:
+                raise ValueError(f"layer {i}: score maps of a head up to 1024 entries together are supported")
         for i, ls in zip(plan.layers, self.specs):
             for b in ls.branches or (ls,):
                 if max(b.dim, b.vdim) > 512:
@@ -120,8 +137,12 @@ class HybridGpuStage(GpuStage):
         else:
             self._attn_of_run = [ls if ls.kind == "attention" else None for ls in self.specs]
         self.gated = spec.norm_kind == "dyt"
+        self.par = spec.parallel_block
         self.runs = spec.layer_runs()
-        if self.gated:
+        if self.par:
+            self.mfma_attn = [False] * len(self.specs)
+            self._load_par(weights, f32, mat)
+        elif self.gated:
             self._load_gated(weights, f32, mat)
         else:
             self.embed = mat(weights.embed)
@@ -173,6 +194,13 @@ class HybridGpuStage(GpuStage):
         self._init_step_state(kv_mem_fraction, decode_states)
         # recurrent state, one slot per row of the block table (the null slot included: padding rows land there)
         self.rec: List[Optional[tuple]] = []
+        for ls in (self.specs if self.par else []):
+            # every layer: the previous token's normed input [slots + 1, H]; a recurrent unit also its convolution's last
+            # inputs and its state, one number per channel
+            st = (torch.zeros(max_slots + 1, spec.hidden_size, device=dev),)
+            if ls.kind == "rglru":
+                st += (torch.zeros(max_slots + 1, max(ls.conv - 1, 1), ls.rec_width, device=dev), torch.zeros(max_slots + 1, ls.rec_width, device=dev))
+            self.rec.append(st)
         for ls in ([spec.layer_specs[li] for li, _ in self.runs] if self.gated else []):
             if ls.kind == "general_delta":
                 self.rec.append((torch.zeros(max_slots + 1, ls.heads, ls.dim, ls.dim, device=dev),))
@@ -180,7 +208,7 @@ class HybridGpuStage(GpuStage):
                 b = ls.branches[1]
                 self.rec.append((torch.zeros(max_slots + 1, b.heads, b.dim, b.vdim + 1, device=dev),
                                  torch.zeros(max_slots + 1, b.heads, 128, device=dev)))
-        for ls in ([] if self.gated else self.specs):
+        for ls in ([] if (self.gated or self.par) else self.specs):
             if ls.kind == "delta":
                 C = 2 * ls.kv_heads * ls.dim + ls.heads * ls.vdim
                 self.rec.append((torch.zeros(max_slots + 1, max(ls.conv - 1, 1), C, device=dev),
@@ -235,6 +263,8 @@ class HybridGpuStage(GpuStage):
 
     # ---- workspaces ---------------------------------------------------------------------------------------
     def _new_work(self, rows: int):
+        if self.par:
+            return self._new_work_par(rows)
         if self.gated:
             return self._new_work_gated(rows)
         s, dev, at = self.spec, self.device, self.act_dtype
@@ -266,11 +296,13 @@ class HybridGpuStage(GpuStage):
     # ---- cache and state sizing -------------------------------------------------------------------------
     def kv_block_bytes(self) -> int:
         e = 4 if self.act_dtype == torch.float32 else 2
+        if self.par:
+            return max(1, sum(BLOCK * e * sum(self._par_rows(ls)) for ls in self.specs if ls.kind != "rglru"))
         return max(1, sum(ls.kv_heads * BLOCK * (ls.dim + ls.vdim) * e for ls in self._attn_of_run if ls is not None))
 
     def _decode_state_bytes(self) -> int:
         n = 0
-        if self.gated:
+        if self.gated or self.par:
             per_row = sum(t.numel() * t.element_size() for t in vars(self.wk0).values() if torch.is_tensor(t)) // self.max_tokens
             return sum(B * (per_row + 4 * self.vocab_pad) for B in self.graph_sizes)
         for B in self.graph_sizes:
@@ -282,6 +314,18 @@ class HybridGpuStage(GpuStage):
     def allocate_kv(self, num_blocks: int):
         dev, at = self.device, self.act_dtype
         self.num_blocks = int(num_blocks)
+        if self.par:
+            # attention: key rows hold a head's score maps side by side, value rows apart; latent attention: ONE row per token,
+            # the normed latent followed by the rotated key part (the values are the row's first entries)
+            self.kv = []
+            for ls in self.specs:
+                if ls.kind == "rglru":
+                    self.kv.append(None)
+                    continue
+                kr, vr = self._par_rows(ls)
+                kc = torch.zeros(self.num_blocks, ls.kv_heads, BLOCK, kr // ls.kv_heads, device=dev, dtype=at)
+                self.kv.append((kc, torch.zeros(self.num_blocks, ls.kv_heads, BLOCK, vr // ls.kv_heads, device=dev, dtype=at) if vr else kc))
+            return
         # zero-filled: a row that was never written must hold finite values
         # (a layer on the MFMA attention kernels keeps K and V slabs of a block side by side, in fragment order)
         self.kv = [None if ls is None else
@@ -314,6 +358,8 @@ class HybridGpuStage(GpuStage):
 
     def _layers(self, wk: _HybridWork, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int, splits: int,
                 alone: bool = False, lead_decode: int = 0):
+        if self.par:
+            return self._layers_par(wk, T, B, tok_pos, tok_seq, q_start, ctx, slots, max_q)
         if self.gated:
             return self._layers_gated(wk, T, B, tok_pos, tok_seq, q_start, ctx, slots, max_q, lead_decode)
         K, eps = self.K, self.spec.norm_eps
@@ -588,6 +634,155 @@ class HybridGpuStage(GpuStage):
                 self.layer_outputs.append(h.clone())
         return None
 
+    # ---- stacks with parallel layers on one norm -----------------------------------------------------------------------
+    @staticmethod
+    def _par_rows(ls) -> tuple:
+        """(entries of a token's key row, of its value row) in the cache of an attention layer, over all its key / value heads."""
+        if ls.kind == "latent_attention":
+            return ls.kv_rank + ls.rot_dim, 0
+        return ls.kv_heads * ls.maps * ls.dim, ls.kv_heads * ls.vdim
+
+    def _load_par(self, weights: StageWeights, f32, mat):
+        """Device weights of a stack with parallel layers. A mixer's input projections are ONE matrix; what a recurrence or a
+        score needs in fp32 (gate matrices, decay rates, norm weights, rotation tables) stays fp32 in both modes."""
+        from .rope import rope_table
+        spec, dev = self.spec, self.device
+        F = torch.nn.functional
+        self.embed, self.lm_head, self.pos_embed = mat(weights.embed), mat(weights.lm_head), None
+        self.lm_head_p = None
+        self.final_norm_w = f32(weights.final_norm_w)
+        self.vocab_pad = packing.padded_n(spec.vocab_size)
+        self.layers = []
+        tables: Dict[tuple, tuple] = {}
+        for i, ls in enumerate(self.specs):
+            l = weights.layers[i]
+            p: Dict[str, object] = {k: f32(l[k]) for k in ("ln1_w", "ls1", "shift")}
+            self._matrix(p, "w_in", mat(l["w_in"]), f32(l["b_in"]) if "b_in" in l else None)
+            self._matrix(p, "w_o", mat(l["w_o"]), None)
+            if ls.rope_dims:
+                key = (ls.rope_dims, ls.rope_base, ls.rope_scaling)
+                if key not in tables:
+                    tables[key] = tuple(t.contiguous() for t in rope_table(ls.rope_dims, ls.rope_base, ls.rope_scaling, self.max_seq_len, dev))
+                p["cos"], p["sin"] = tables[key]
+            else:
+                p["cos"] = p["sin"] = None
+            if ls.kind == "rglru":
+                p["conv_w"], p["conv_b"] = f32(l["conv_w"]), f32(l["conv_b"])
+                # per block the decay gate's rows, then the input gate's: one block-diagonal product gives both
+                p["w_g"] = torch.cat([f32(l["w_ra"]), f32(l["w_ri"])], dim=1).contiguous()
+                p["b_g"] = torch.cat([f32(l["b_ra"]), f32(l["b_ri"])], dim=1).reshape(-1).contiguous()
+                p["clam"] = (8.0 * F.softplus(f32(l["lam"]))).contiguous()
+            elif ls.kind == "attention":
+                lq1, lk1, lq2, lk2 = (f32(l[k]) for k in ("lq1", "lk1", "lq2", "lk2"))
+                p["lam"] = float(torch.exp((lq1 * lk1).sum()) - torch.exp((lq2 * lk2).sum()) + ls.diff) if ls.maps == 2 else 0.0
+            else:
+                H, d, dr, dv, R = ls.heads, ls.dim, ls.rot_dim, ls.vdim, ls.kv_rank
+                p["dq_norm"], p["dkv_norm"] = f32(l["dq_norm"]), f32(l["dkv_norm"])
+                self._matrix(p, "w_uq", mat(l["w_uq"]), None)
+                # per head: q . (W_uk c) = (W_uk^T q) . c, so the key up-projection moves to the query's side (the rotated
+                # entries pass through an identity) and the cache keeps the latent alone
+                wa = torch.zeros(H, R + dr, d + dr, device=dev, dtype=self.act_dtype)
+                wa[:, :R, :d] = mat(l["w_uk"]).reshape(H, d, R).transpose(1, 2)
+                wa[:, R:, d:] = torch.eye(dr, device=dev, dtype=self.act_dtype)
+                p["w_abs"], p["w_uv"] = wa.contiguous(), mat(l["w_uv"]).reshape(H, dv, R).contiguous()
+            if ls.ff:
+                p["ls2"] = f32(l["ls2"])
+                self._matrix(p, "w_up", mat(l["w_up"]), None)
+                self._matrix(p, "w_down", mat(l["w_down"]), None)
+                a = f32(l["act"]).reshape(-1)
+                p["pq"] = torch.stack([F.softplus(a[0]), 0.5 + F.softplus(a[1])]).contiguous()
+            self.layers.append(p)
+            weights.layers[i] = {}
+        if self._packed and spec.hidden_size % 128 == 0:
+            self.lm_head_p = packing.pack_weight(self.lm_head)
+            self._shapes.append((self.vocab_pad, spec.hidden_size, False))
+
+    def _new_work_par(self, rows: int):
+        s, dev, at = self.spec, self.device, self.act_dtype
+        z = lambda n, dt=torch.float32: torch.zeros(max(int(n), 1), device=dev, dtype=dt)
+        B, H = min(rows, self.max_batch), s.hidden_size
+        zc = uc = mc = yc = z2 = ac = cq = q32 = q16 = qa = ol = 1
+        for ls, p in zip(self.specs, self.layers):
+            zc, yc = max(zc, self._cols(p, "w_in")), max(yc, self._cols(p, "w_o"))
+            if ls.kind == "rglru":
+                uc, mc = max(uc, ls.rec_width), max(mc, ls.rec_width)
+            else:
+                mc = max(mc, ls.heads * ls.vdim)
+            if ls.kind == "latent_attention":
+                cq, q32 = max(cq, ls.q_rank), max(q32, self._cols(p, "w_uq"))
+                q16, qa = max(q16, ls.heads * (ls.dim + ls.rot_dim)), max(qa, ls.heads * (ls.kv_rank + ls.rot_dim))
+                ol = max(ol, ls.heads * ls.kv_rank)
+            if ls.ff:
+                z2, ac, yc = max(z2, self._cols(p, "w_up")), max(ac, ls.ff), max(yc, self._cols(p, "w_down"))
+        ws_floats = self._ws_floats
+        if self._packed and rows > self.decode_rows:
+            for m_ in {rows, min(rows, 512), min(rows, 1024)}:
+                if m_ > self.decode_rows:
+                    ws_floats = max([ws_floats] + [int(self.K.gemm_ws_floats(m_, n_, k_)) for n_, k_, _ in self._shapes])
+        return SimpleNamespace(
+            h=torch.zeros(rows, H, device=dev), n32=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at),
+            xs=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc), u=z(rows * uc), gates=z(rows * 2 * uc), mixed=z(rows * mc, at),
+            ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2), act=z(rows * ac, at), cq=z(rows * cq, at), q32=z(rows * q32),
+            q16=z(rows * q16, at), qa=z(rows * qa), olat=z(rows * ol, at), ws=z(ws_floats + 4096),
+            head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
+
+    def _layers_par(self, wk, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int):
+        K, eps, H = self.K, self.spec.norm_eps, self.spec.hidden_size
+        h, n32, xn, xs = wk.h[:T], wk.n32[:T], wk.xn[:T], wk.xs[:T]
+        view = lambda buf, cols: buf[:T * cols].view(T, cols)
+        keep = self.keep_layer_outputs and not torch.cuda.is_current_stream_capturing()
+        if keep:
+            self.layer_outputs = []
+        table, n_layers = self.block_table, len(self.layers)
+        K.par_norm(xn, n32, h, None, None, None, None, self.layers[0]["ln1_w"], None, tok_seq, eps)
+        for li, (ls, p) in enumerate(zip(self.specs, self.layers)):
+            K.token_shift(xs, n32, self.rec[li][0], p["shift"], tok_pos, tok_seq)
+            z = view(wk.z, self._cols(p, "w_in"))
+            self._mm(wk, z, xs, p, "w_in")
+            if ls.kind == "rglru":
+                W, bw = ls.rec_width, ls.rec_width // ls.blocks
+                u, gates, mixed = view(wk.u, W), view(wk.gates, 2 * W), view(wk.mixed, W)
+                K.short_conv_act(u, z[:, W:2 * W], self.rec[li][1], p["conv_w"], p["conv_b"], q_start, ctx, slots, max_q, False)
+                K.gemm_blocks(gates, u, p["w_g"], p["b_g"], bw, 2 * bw)
+                K.rglru_scan(mixed, u, gates, z[:, :W], p["clam"], self.rec[li][2], q_start, ctx, slots, bw, max_q)
+            elif ls.kind == "attention":
+                Hh, G, d, dv, M = ls.heads, ls.kv_heads, ls.dim, ls.vdim, ls.maps
+                qn, kn, vn = Hh * M * d, G * M * d, G * dv
+                kc, vc = self.kv[li]
+                mixed = view(wk.mixed, Hh * dv)
+                K.rope_cache_write(z, Hh * M, d, 0, None, 0, z[:, qn:], kn, G * M, d, 0, vn, kc, vc, ls.rope_dims, ls.rope_interleaved,
+                                   p["cos"], p["sin"], tok_pos, tok_seq, table)
+                K.multi_attention(mixed, z, M * d, kc, vc, 0, tok_pos, tok_seq, table, Hh, d, dv, M, ls.scale, ls.window or 0,
+                                  ls.keep_first, ls.softcap, p["lam"], 1.0 - ls.diff, eps,
+                                  z[:, qn + kn + vn:qn + kn + vn + Hh * dv] if ls.out_gate else None)
+            else:
+                Hh, d, dr, dv, R, qr = ls.heads, ls.dim, ls.rot_dim, ls.vdim, ls.kv_rank, ls.q_rank
+                kc = self.kv[li][0]
+                cq, q32 = view(wk.cq, qr), view(wk.q32, self._cols(p, "w_uq"))
+                q16, qa, olat, mixed = view(wk.q16, Hh * (d + dr)), view(wk.qa, Hh * (R + dr)), view(wk.olat, Hh * R), view(wk.mixed, Hh * dv)
+                K.norm32(cq, z[:, :qr], None, None, p["dq_norm"], None, eps, 0.0)
+                K.norm32(z[:, qr:qr + R], z[:, qr:qr + R], None, None, p["dkv_norm"], None, eps, 0.0)       # (in place)
+                self._mm(wk, q32, cq, p, "w_uq")
+                K.rope_cache_write(q32, Hh, d + dr, d, q16, Hh * (d + dr), z[:, qr:], R + dr, 1, R + dr, R, 0, kc, None, ls.rope_dims,
+                                   ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
+                K.gemm_blocks(qa, q16, p["w_abs"], None, d + dr, R + dr)
+                K.multi_attention(olat, qa, R + dr, kc, kc, 0, tok_pos, tok_seq, table, Hh, R + dr, R, 1, ls.scale, 0, 0, 0.0, 0.0, 1.0,
+                                  eps, None)
+                K.gemm_blocks(mixed, olat, p["w_uv"], None, R, dv)
+            ya, yb = view(wk.ya, self._cols(p, "w_o")), None
+            self._mm(wk, ya, mixed, p, "w_o")
+            if ls.ff:
+                z2, act, yb = view(wk.z2, self._cols(p, "w_up")), view(wk.act, ls.ff), view(wk.yb, self._cols(p, "w_down"))
+                self._mm(wk, z2, xn, p, "w_up")
+                K.xielu(act, z2, p["pq"])
+                self._mm(wk, yb, act, p, "w_down")
+                yb = yb[:, :H]
+            nxt = self.layers[li + 1]["ln1_w"] if li + 1 < n_layers else None
+            K.par_norm(xn if nxt is not None else None, n32, h, ya[:, :H], yb, p["ls1"], p.get("ls2"), nxt, self.rec[li][0], tok_seq, eps)
+            if keep:
+                self.layer_outputs.append(h.clone())
+        return None
+
     def _fold(self, wk, T: int, pend):
         return None
 
@@ -597,6 +792,8 @@ class HybridGpuStage(GpuStage):
         if self.gated:
             K.dyt_gate(hx, wk.h[:T], None, None, None, None, None, None, None, self.final_norm_w, self.final_norm_b, rows_idx[:R],
                        self.final_norm_a, self.spec.norm_eps)
+        elif self.par:
+            K.norm32(hx, wk.h[:T], None, None, self.final_norm_w, rows_idx[:R], self.spec.norm_eps, 0.0)
         else:
             K.norm32(hx, wk.h[:T], None, None, self.final_norm_w, rows_idx[:R], self.spec.norm_eps, 1.0)
         if self.lm_head_p is not None:
@@ -605,6 +802,8 @@ class HybridGpuStage(GpuStage):
             K.gemm_any(wk.logits[:R, :self.spec.vocab_size], hx, self.lm_head, None, 0)
         if self.spec.logit_softcap > 0:
             K.softcap(wk.logits[:R], self.spec.vocab_size, self.spec.logit_softcap)
+        if self.spec.logit_scale != 1.0:
+            K.scale_rows(wk.logits[:R], self.spec.vocab_size, self.spec.logit_scale)
         return wk.logits[:R]
 
     def memory_report(self) -> Dict[str, float]:

@@ -708,7 +708,8 @@ void embed32(Tensor out, const Tensor& ids, const Tensor& table) {
 void norm32(const std::optional<Tensor>& out, Tensor x, OptTensor y, OptTensor wb, OptTensor wn, OptTensor row_idx, double eps,
             double off) {
   DLIA_ON_DEVICE_OF(x);
-  check_f32(x, "x"); check_mat(x, "x");
+  check_mat(x, "x");                       // (rows may be a column slice of a wider buffer: the row stride is passed on)
+  DLIA_CHECK(x.scalar_type() == at::kFloat, "x must be float32");
   const int64_t H = x.size(1);
   int64_t rows = x.size(0);
   const int* ridx = nullptr;
@@ -823,8 +824,8 @@ void window_attention(Tensor out, const Tensor& qkv, const Tensor& kcache, const
                         cur_stream());
 }
 
-void short_conv(Tensor y, const Tensor& z, Tensor carry, const Tensor& taps, const Tensor& q_start, const Tensor& ctx,
-                const Tensor& slots, int64_t max_q) {
+void short_conv_act(Tensor y, const Tensor& z, Tensor carry, const Tensor& taps, OptTensor bias, const Tensor& q_start,
+                    const Tensor& ctx, const Tensor& slots, int64_t max_q, bool silu) {
   DLIA_ON_DEVICE_OF(y);
   check_f32(y, "y"); check_f32(carry, "carry"); check_f32(taps, "taps"); check_mat(z, "z");
   DLIA_CHECK(z.is_cuda() && z.scalar_type() == at::kFloat, "z: float32");
@@ -837,7 +838,12 @@ void short_conv(Tensor y, const Tensor& z, Tensor carry, const Tensor& taps, con
   DLIA_CHECK(max_q <= y.size(0), "short_conv: max_q beyond the step's tokens");
   dlia_short_conv(y.data_ptr<float>(), z.data_ptr<float>(), carry.data_ptr<float>(), taps.data_ptr<float>(), q_start.data_ptr<int>(),
                   ctx.data_ptr<int>(), slots.data_ptr<int>(), (int)B, (int)max_q, (int)C, (int)K, z.stride(0), (int)carry.size(0),
-                  cur_stream());
+                  opt_f32(bias, C, "bias"), silu ? 1 : 0, cur_stream());
+}
+
+void short_conv(Tensor y, const Tensor& z, Tensor carry, const Tensor& taps, const Tensor& q_start, const Tensor& ctx,
+                const Tensor& slots, int64_t max_q) {
+  short_conv_act(y, z, carry, taps, std::nullopt, q_start, ctx, slots, max_q, true);
 }
 
 void unit_heads(Tensor x, int64_t heads, int64_t d, int64_t scaled_heads, double mult, double eps) {
@@ -882,6 +888,7 @@ TORCH_LIBRARY(dlia, m) {
   m.def("kv_store(Tensor qkv, Tensor(a!)? vfirst, Tensor? lam, int mix, Tensor(b!) kcache, Tensor(c!) vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int G, int d, int dv, int q_cols) -> ()");
   m.def("window_attention(Tensor(a!) out, Tensor qkv, Tensor kcache, Tensor vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int G, int d, int dv, float scale, int window, bool sink) -> ()");
   m.def("short_conv(Tensor(a!) y, Tensor z, Tensor(b!) carry, Tensor taps, Tensor q_start, Tensor ctx, Tensor slots, int max_q) -> ()");
+  m.def("short_conv_act(Tensor(a!) y, Tensor z, Tensor(b!) carry, Tensor taps, Tensor? bias, Tensor q_start, Tensor ctx, Tensor slots, int max_q, bool silu) -> ()");
   m.def("unit_heads(Tensor(a!) x, int heads, int d, int scaled_heads, float mult, float eps) -> ()");
   m.def("delta_rule(Tensor(a!) o, Tensor y, Tensor z, Tensor(b!) state, Tensor A_log, Tensor dt_bias, Tensor q_start, Tensor ctx, Tensor slots, int G, int Hv, int d, int dv, int col_beta, int col_a, int max_q) -> ()");
   m.def("norm(Tensor(a!) out, Tensor(b!) x, Tensor? delta, Tensor? partial, int splits, Tensor? pbias, Tensor w, Tensor? b, Tensor? row_idx, float eps, int mode) -> ()");
@@ -921,6 +928,7 @@ TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
   m.impl("kv_store", &kv_store);
   m.impl("window_attention", &window_attention);
   m.impl("short_conv", &short_conv);
+  m.impl("short_conv_act", &short_conv_act);
   m.impl("unit_heads", &unit_heads);
   m.impl("delta_rule", &delta_rule);
   m.impl("norm", &norm);

@@ -6,7 +6,7 @@
 // owns state slot slots[b]. A sequence's first step (ctx = 0) starts from zeros whatever its slot held before,
 // so a slot needs no clearing when it changes hands; later steps continue from the slot.
 //
-//   short_conv      y[t, c] = silu(sum_j taps[c, j] * x[t - (K-1-j), c]); inputs before the step come from the
+//   short_conv      y[t, c] = act(bias[c] + sum_j taps[c, j] * x[t - (K-1-j), c]), act = silu or none, bias optional; inputs before the step come from the
 //                   slot's K-1 carried inputs, inputs before the sequence's start are zero
 //   conv_carry      the slot's carried inputs become the last K-1 inputs including this step's (runs after
 //                   short_conv has read the old ones)
@@ -27,7 +27,7 @@ constexpr int kConvMaxTaps = 16;
 __global__ __launch_bounds__(256) void short_conv_kernel(
     float* __restrict__ y, const float* __restrict__ z, const float* __restrict__ carry, const float* __restrict__ taps,
     const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots, int C, int K, long ldz,
-    int tokb, int state_rows) {
+    int tokb, int state_rows, const float* __restrict__ bias, int silu) {
   const int b = blockIdx.x;
   const int t0 = q_start[b], n = q_start[b + 1] - t0, c0 = ctx[b], slot = slots[b];
   const int r0 = blockIdx.y * tokb, r1 = min(n, r0 + tokb);
@@ -37,8 +37,9 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
     float w[kConvMaxTaps];
 #pragma unroll
     for (int j = 0; j < kConvMaxTaps; ++j) w[j] = j < K ? taps[(long)c * K + j] : 0.f;
+    const float bc = bias ? bias[c] : 0.f;
     for (int r = r0; r < r1; ++r) {
-      float acc = 0.f;
+      float acc = bc;
 #pragma unroll
       for (int j = 0; j < kConvMaxTaps; ++j) {
         if (j >= K) break;
@@ -48,7 +49,7 @@ __global__ __launch_bounds__(256) void short_conv_kernel(
         else x = (c0 + s >= 0) ? st[(long)(K - 1 + s) * C + c] : 0.f;
         acc += w[j] * x;
       }
-      y[(long)(t0 + r) * C + c] = acc / (1.f + expf(-acc));
+      y[(long)(t0 + r) * C + c] = silu ? acc / (1.f + expf(-acc)) : acc;
     }
   }
 }
@@ -267,12 +268,13 @@ __global__ __launch_bounds__(DECODE ? 64 : 128) void delta_rule_kernel(
 }  // namespace dlia
 
 extern "C" void dlia_short_conv(float* y, const float* z, float* carry, const float* taps, const int* q_start, const int* ctx,
-                                const int* slots, int B, int max_q, int C, int K, long ldz, int state_rows, hipStream_t stream) {
+                                const int* slots, int B, int max_q, int C, int K, long ldz, int state_rows, const float* bias,
+                                int silu, hipStream_t stream) {
   if (B <= 0 || max_q <= 0) return;
   // a workgroup takes 8 tokens of a sequence and every fourth 256-channel slice (thousands of workgroups for a prompt portion)
   const int tokb = 8, cblocks = (C + 1023) / 1024 < 1 ? 1 : (C + 1023) / 1024;
   hipLaunchKernelGGL(dlia::short_conv_kernel, dim3(B, (max_q + tokb - 1) / tokb, cblocks), dim3(256), 0, stream, y, z, carry, taps,
-                     q_start, ctx, slots, C, K, ldz, tokb, state_rows);
+                     q_start, ctx, slots, C, K, ldz, tokb, state_rows, bias, silu);
   if (K > 1)
     hipLaunchKernelGGL(dlia::conv_carry_kernel, dim3(B, (C + 255) / 256), dim3(256), 0, stream, carry, z, q_start, ctx, slots, C,
                        K, ldz, state_rows);

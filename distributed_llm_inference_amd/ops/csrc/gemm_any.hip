@@ -27,8 +27,11 @@ __device__ __forceinline__ float gelu_tanh_exact(float x) {
 template <typename T, typename OT, int EPI>
 __global__ __launch_bounds__(256) void gemm_any_kernel(OT* __restrict__ C, const T* __restrict__ A, const T* __restrict__ W,
                                                        const float* __restrict__ bias, int M, int N, int K, long lda,
-                                                       long ldw, long ldc, int vec_ok) {
+                                                       long ldw, long ldc, int vec_ok, long a_step, long w_step, long c_step) {
   constexpr int VEC = 16 / sizeof(T), KS = 4 * VEC;
+  // (blockIdx.z: one of several independent products of equal shape, e.g. the blocks of a block-diagonal matrix)
+  A += blockIdx.z * a_step; W += blockIdx.z * w_step; C += blockIdx.z * c_step;
+  if (bias) bias += (long)blockIdx.z * N;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int m_base = blockIdx.y * 64 + (wave >> 1) * 32, n_base = blockIdx.x * 64 + (wave & 1) * 32;
   if (m_base >= M || n_base >= N) return;
@@ -97,16 +100,17 @@ __global__ __launch_bounds__(256) void gated_gelu_kernel(bf16* __restrict__ act,
 
 template <typename T, typename OT>
 static void launch_any(void* C, const void* A, const void* W, const float* bias, int M, int N, int K, long lda, long ldw,
-                       long ldc, int epi, hipStream_t stream) {
+                       long ldc, int epi, hipStream_t stream, int blocks = 1, long a_step = 0, long w_step = 0, long c_step = 0) {
   constexpr int VEC = 16 / sizeof(T);
-  const int vec_ok = K % VEC == 0 && lda % VEC == 0 && ldw % VEC == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0;
-  const dim3 grid((N + 63) / 64, (M + 63) / 64);
+  const int vec_ok = K % VEC == 0 && lda % VEC == 0 && ldw % VEC == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 &&
+                     a_step % VEC == 0 && w_step % VEC == 0;
+  const dim3 grid((N + 63) / 64, (M + 63) / 64, blocks);
   if (epi == 0)
     hipLaunchKernelGGL((gemm_any_kernel<T, OT, 0>), grid, dim3(256), 0, stream, (OT*)C, (const T*)A, (const T*)W, bias, M, N,
-                       K, lda, ldw, ldc, vec_ok);
+                       K, lda, ldw, ldc, vec_ok, a_step, w_step, c_step);
   else
     hipLaunchKernelGGL((gemm_any_kernel<T, OT, 1>), grid, dim3(256), 0, stream, (OT*)C, (const T*)A, (const T*)W, bias, M, N,
-                       K, lda, ldw, ldc, vec_ok);
+                       K, lda, ldw, ldc, vec_ok, a_step, w_step, c_step);
 }
 
 }  // namespace dlia
@@ -127,4 +131,16 @@ extern "C" void dlia_gemm_any(void* C, int out_f32, const void* A, const void* W
     dlia::launch_any<dlia::bf16, float>(C, A, W, bias, M, N, K, lda, ldw, ldc, epi, stream);
   else
     dlia::launch_any<dlia::bf16, dlia::bf16>(C, A, W, bias, M, N, K, lda, ldw, ldc, epi, stream);
+}
+
+extern "C" void dlia_gemm_blocks(void* C, int out_f32, const void* A, const void* W, int in_f32, const float* bias, int M, int N,
+                                 int K, long lda, long ldw, long ldc, int blocks, long a_step, long w_step, long c_step,
+                                 hipStream_t stream) {
+  if (M <= 0 || N <= 0 || blocks <= 0) return;
+  if (in_f32)
+    dlia::launch_any<float, float>(C, A, W, bias, M, N, K, lda, ldw, ldc, 0, stream, blocks, a_step, w_step, c_step);
+  else if (out_f32)
+    dlia::launch_any<dlia::bf16, float>(C, A, W, bias, M, N, K, lda, ldw, ldc, 0, stream, blocks, a_step, w_step, c_step);
+  else
+    dlia::launch_any<dlia::bf16, dlia::bf16>(C, A, W, bias, M, N, K, lda, ldw, ldc, 0, stream, blocks, a_step, w_step, c_step);
 }

@@ -118,6 +118,10 @@ void dlia_gated_headnorm(void* out, int out_f32, const float* o, const float* ga
 // gelu_tanh(gate) * up, N / 2 columns
 void dlia_gemm_any(void* C, int out_f32, const void* A, const void* W, int in_f32, const float* bias, int M, int N, int K,
                    long lda, long ldw, long ldc, int epi, hipStream_t stream);
+// `blocks` independent products in one launch: block b reads A + b * a_step, W + b * w_step, bias + b * N and writes
+// C + b * c_step (steps in elements). epi 0 only.
+void dlia_gemm_blocks(void* C, int out_f32, const void* A, const void* W, int in_f32, const float* bias, int M, int N, int K,
+                      long lda, long ldw, long ldc, int blocks, long a_step, long w_step, long c_step, hipStream_t stream);
 
 // act[m, j] = gelu_tanh(gu[m, j]) * gu[m, F + j] (bf16, F a multiple of 8, 16-byte aligned rows)
 void dlia_gated_gelu(void* act, const void* gu, int M, int F, long ldg, long lda, hipStream_t stream);
@@ -137,7 +141,8 @@ void dlia_value_mix(void* qkv, float* vfirst, const float* lam, int mix, int T, 
 
 // ---- delta_rule.hip -------------------------------------------------------------------------
 void dlia_short_conv(float* y, const float* z, float* carry, const float* taps, const int* q_start, const int* ctx,
-                     const int* slots, int B, int max_q, int C, int K, long ldz, int state_rows, hipStream_t stream);
+                     const int* slots, int B, int max_q, int C, int K, long ldz, int state_rows, const float* bias, int silu,
+                     hipStream_t stream);
 void dlia_unit_heads(float* x, int T, int heads, int d, long ld, int scaled_heads, float mult, float eps, hipStream_t stream);
 int dlia_delta_rule(float* o, const float* y, const float* z, float* state, const float* A_log, const float* dt_bias,
                     const int* q_start, const int* ctx, const int* slots, int B, int G, int Hv, int d, int dv, int C, long ldz,
@@ -175,6 +180,28 @@ void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int
 void dlia_moe_combine(float* out, const float* y, const int* pair_row, const float* wts, int T, int H, int top, long ldo,
                       hipStream_t stream);
 
+
+// ---- parallel_ops.hip (parallel layers on one norm, token shift, rotation + cache write, attention over score maps, RG-LRU) ----
+void dlia_par_norm(void* out, int out_f32, float* out32, float* x, const float* ya, const float* yb, const float* ls1,
+                   const float* ls2, const float* w, float* carry, const int* tok_seq, int T, int state_rows, int H, long ldx,
+                   long ldya, long ldyb, long ldo, float eps, hipStream_t stream);
+void dlia_token_shift(void* out, int out_f32, const float* n32, const float* carry, const float* mu, const int* tok_pos,
+                      const int* tok_seq, int T, int state_rows, int H, long ldo, hipStream_t stream);
+void dlia_rope_cache_write(float* q, long ldq, int q_vecs, int q_stride, int q_off, void* q_out, long ldqo, int q_cols, float* kv,
+                           long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols, void* kcache, void* vcache,
+                           int f32, int G, int dims, int interleaved, const float* cos_t, const float* sin_t, int table_pos,
+                           const int* tok_pos, const int* tok_seq, const int* block_table, int T, int max_blocks, int num_blocks,
+                           int table_rows, hipStream_t stream);
+void dlia_multi_attention(void* out, long ldo, const float* q, long ldq, int q_head, const void* kcache, int k_row,
+                          const void* vcache, int v_row, int v_off, int f32, const int* tok_pos, const int* tok_seq,
+                          const int* block_table, int T, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
+                          int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
+                          const float* gate, long ldg, hipStream_t stream);
+void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg, const float* ypre,
+                     long ldy, const float* clam, float* state, const int* q_start, const int* ctx, const int* slots, int B,
+                     int max_q, int W, int bw, int state_rows, hipStream_t stream);
+void dlia_xielu(void* act, int out_f32, const float* z, int M, int F, long ldz, long lda, const float* pq, hipStream_t stream);
+void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStream_t stream);
 // ---- misc.hip -------------------------------------------------------------------------
 void dlia_advance_i32(int* x, int n, int delta, hipStream_t stream);
 void dlia_scatter_rows_i32(int* dst, const int* rows, const int* src, int nrows, int ncols, int dst_rows, hipStream_t stream);

@@ -1,0 +1,483 @@
+// Kernels for stacks whose layers run their two sublayers side by side on ONE norm of an fp32 residual stream,
+//     n = rms(x) w;   x <- x + ls1 * mixer(shifted(n)) + ls2 * ff(n),
+// whose mixers read a blend of n with the previous token's n, and whose mixers are a real-gated linear recurrence,
+// attention over one or two score maps per head with partial rotation, or attention through a cached latent.
+//
+//   par_norm        one launch per layer boundary: the carried n of the closing layer is saved for its sequences' next
+//                   step, x += ls1 * ya + ls2 * yb, and the next layer's n leaves in fp32 (for the blend) and in the
+//                   GEMMs' input type (for the feed-forward)
+//   token_shift     n + (previous n - n) * mu per token; the previous n is the row above, the slot's carried n at the
+//                   start of a portion, zeros at position 0
+//   rope_cache_write per token: rotates the first `dims` entries of a set of q vectors and of the k vectors (pairs
+//                   (2i, 2i + 1) or (i, i + dims / 2), angles from a table by position), optionally leaves q in the
+//                   GEMMs' input type, and writes the k row (and the v row) into the paged cache
+//   multi_attention one wave per (token, head): softmax attention over the paged cache with a window that also keeps
+//                   the sequence's first tokens, scores through cap tanh(s / cap); with two maps per head both are
+//                   walked at once over the shared values and combined as rms(a1 - lam a2) (1 - diff) sigmoid(gate).
+//                   Keys are rows of any length (a map is a slice of the row), values may be a slice of the key rows.
+//   rglru_scan      S <- a S + sqrt(1 - a^2) i u per channel with a = exp(-c r), r and i sigmoids of the block gates;
+//                   read-out S * gelu_tanh(y). Long portions are cut into segments that are scanned side by side and
+//                   joined through the segments' (decay product, offset) pairs.
+//   xielu, scale_rows   the feed-forward's activation; logits times a constant
+// Everything is fp32 except what feeds a GEMM or sits in the cache (the compute type, bf16 or fp32).
+#include "common.h"
+#include "launch.h"
+
+namespace dlia {
+
+constexpr int kParBlock = 32;        // tokens per cache block
+constexpr int kParThreads = 256;
+
+// ---- norm / residual / carried rows -------------------------------------------------------------------------------
+template <typename OT>
+__global__ __launch_bounds__(kParThreads) void par_norm_kernel(
+    OT* __restrict__ out, float* __restrict__ out32, float* __restrict__ x, const float* __restrict__ ya,
+    const float* __restrict__ yb, const float* __restrict__ ls1, const float* __restrict__ ls2, const float* __restrict__ w,
+    float* __restrict__ carry, const int* __restrict__ tok_seq, int T, int state_rows, int H, long ldx, long ldya, long ldyb,
+    long ldo, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  float* xr = x + (long)t * ldx;
+  float* nr = out32 + (long)t * H;
+  if (carry) {
+    const int slot = tok_seq[t];
+    const bool last = t + 1 == T || tok_seq[t + 1] != slot;
+    if (last && slot >= 0 && slot < state_rows)
+      for (int i = threadIdx.x; i < H; i += kParThreads) carry[(long)slot * H + i] = nr[i];
+  }
+  if (ya) {
+    const float* ar = ya + (long)t * ldya;
+    const float* br = yb ? yb + (long)t * ldyb : nullptr;
+    for (int i = threadIdx.x; i < H; i += kParThreads) {
+      float add = ls1[i] * ar[i];
+      if (br) add += ls2[i] * br[i];
+      xr[i] += add;
+    }
+  }
+  if (!out) return;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < H; i += kParThreads) { const float v = xr[i]; s += v * v; }   // (each thread re-reads what it wrote itself)
+  s = block_sum(s, scratch);
+  const float r = 1.f / sqrtf(s / H + eps);
+  OT* orow = out + (long)t * ldo;
+  for (int i = threadIdx.x; i < H; i += kParThreads) {
+    const float v = xr[i] * r * w[i];
+    nr[i] = v;
+    orow[i] = (OT)v;
+  }
+}
+
+template <typename OT>
+__global__ __launch_bounds__(kParThreads) void token_shift_kernel(
+    OT* __restrict__ out, const float* __restrict__ n32, const float* __restrict__ carry, const float* __restrict__ mu,
+    const int* __restrict__ tok_pos, const int* __restrict__ tok_seq, int state_rows, int H, long ldo) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t], slot = tok_seq[t];
+  const float* cur = n32 + (long)t * H;
+  const float* prev = nullptr;
+  if (pos > 0) {
+    if (t > 0 && tok_seq[t - 1] == slot && tok_pos[t - 1] == pos - 1) prev = cur - H;
+    else if (slot >= 0 && slot < state_rows) prev = carry + (long)slot * H;
+  }
+  OT* orow = out + (long)t * ldo;
+  for (int i = threadIdx.x; i < H; i += kParThreads) {
+    const float h = cur[i], p = prev ? prev[i] : 0.f;
+    orow[i] = (OT)(h + (p - h) * mu[i]);
+  }
+}
+
+// ---- rotation + cache write ----------------------------------------------------------------------------------------
+// A set of vectors inside a row: entries [off, off + dims) of every `stride` entries are rotated.
+__device__ __forceinline__ void rotate_row(float* row, int n_vec, int stride, int off, int dims, int interleaved,
+                                           const float* cs, const float* sn) {
+  const int half = dims >> 1;
+  for (int p = threadIdx.x; p < n_vec * half; p += kParThreads) {
+    const int vi = p / half, pi = p % half;
+    float* v = row + (long)vi * stride + off;
+    const int i0 = interleaved ? 2 * pi : pi, i1 = interleaved ? 2 * pi + 1 : pi + half;
+    const float a = v[i0], b = v[i1], c = cs[pi], s = sn[pi];
+    v[i0] = a * c - b * s;
+    v[i1] = b * c + a * s;
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kParThreads) void rope_cache_write_kernel(
+    float* __restrict__ q, long ldq, int q_vecs, int q_stride, int q_off, T* __restrict__ q_out, long ldqo, int q_cols,
+    float* __restrict__ kv, long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols, T* __restrict__ kcache,
+    T* __restrict__ vcache, int G, int dims, int interleaved, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    int table_pos, const int* __restrict__ tok_pos, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
+    int max_blocks, int num_blocks, int table_rows) {
+  const int t = blockIdx.x;
+  const int pos = tok_pos[t], slot = tok_seq[t];
+  float* qrow = q + (long)t * ldq;
+  float* krow = kv + (long)t * ldkv;
+  if (dims > 0 && pos >= 0 && pos < table_pos) {
+    const float* cs = cos_t + (long)pos * (dims >> 1);
+    const float* sn = sin_t + (long)pos * (dims >> 1);
+    rotate_row(qrow, q_vecs, q_stride, q_off, dims, interleaved, cs, sn);
+    rotate_row(krow, k_vecs, k_stride, k_off, dims, interleaved, cs, sn);
+  }
+  __syncthreads();
+  if (q_out)
+    for (int i = threadIdx.x; i < q_cols; i += kParThreads) q_out[(long)t * ldqo + i] = (T)qrow[i];
+  int blk = -1;
+  if (slot >= 0 && slot < table_rows && pos >= 0 && pos / kParBlock < max_blocks) blk = block_table[(long)slot * max_blocks + pos / kParBlock];
+  if (blk < 0 || blk >= num_blocks) return;
+  const int off = pos % kParBlock, dk = k_cols / G;
+  for (int i = threadIdx.x; i < k_cols; i += kParThreads) {
+    const int g = i / dk, c = i % dk;
+    kcache[(((long)blk * G + g) * kParBlock + off) * dk + c] = (T)krow[i];
+  }
+  if (vcache) {
+    const int dv = v_cols / G;
+    const float* vrow = krow + k_cols;
+    for (int i = threadIdx.x; i < v_cols; i += kParThreads) {
+      const int g = i / dv, c = i % dv;
+      vcache[(((long)blk * G + g) * kParBlock + off) * dv + c] = (T)vrow[i];
+    }
+  }
+}
+
+// ---- attention ---------------------------------------------------------------------------------------------------
+constexpr int kMultiMaxQ = 1024;     // MAPS * d
+constexpr int kMultiMaxDV = 512;
+
+__device__ __forceinline__ float dot_row(const float* qs, const bf16* k, int d, bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int i = 0; i < d; i += 8) {
+      float f[8];
+      unpack8(ld16(k + i), f);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc += qs[i + j] * f[j];
+    }
+  } else {
+    for (int i = 0; i < d; ++i) acc += qs[i] * (float)k[i];
+  }
+  return acc;
+}
+__device__ __forceinline__ float dot_row(const float* qs, const float* k, int d, bool vec) {
+  float acc = 0.f;
+  if (vec) {
+    for (int i = 0; i < d; i += 4) {
+      const f32x4 f = *reinterpret_cast<const f32x4*>(k + i);
+      acc += qs[i] * f[0] + qs[i + 1] * f[1] + qs[i + 2] * f[2] + qs[i + 3] * f[3];
+    }
+  } else {
+    for (int i = 0; i < d; ++i) acc += qs[i] * k[i];
+  }
+  return acc;
+}
+
+template <typename T, typename OT, int MAPS>
+__global__ __launch_bounds__(256) void multi_attention_kernel(
+    OT* __restrict__ out, long ldo, const float* __restrict__ q, long ldq, int q_head, const T* __restrict__ kcache, int k_row,
+    const T* __restrict__ vcache, int v_row, int v_off, const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
+    const int* __restrict__ block_table, int items, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
+    float scale, int window, int keep_first, float softcap, float lam, float post, float eps, const float* __restrict__ gate,
+    long ldg, int vec) {
+  __shared__ float qs[4][kMultiMaxQ];
+  const int wave = threadIdx.x >> 6, lane = lane_id();
+  const int item = blockIdx.x * 4 + wave;
+  if (item >= items) return;
+  const int t = item / H, h = item % H, g = h / (H / G);
+  const int pos = tok_pos[t], slot = tok_seq[t];
+  OT* orow = out + (long)t * ldo + (long)h * dv;
+  const bool live = slot >= 0 && slot < table_rows && pos >= 0 && pos / kParBlock < max_blocks;
+  if (!live) {                                   // padding row of a fixed-shape step
+    for (int c = lane; c < dv; c += 64) orow[c] = (OT)0.f;
+    return;
+  }
+  const float* qrow = q + (long)t * ldq + (long)h * q_head;
+  for (int i = lane; i < MAPS * d; i += 64) qs[wave][i] = qrow[i] * scale;
+  __builtin_amdgcn_wave_barrier();
+  const int* table = block_table + (long)slot * max_blocks;
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int kept = (window > 0 && keep_first > 0) ? min(keep_first, lo) : 0;    // keys [0, kept) in front of the window
+  float m[MAPS], l[MAPS], acc[MAPS][kMultiMaxDV / 64];
+#pragma unroll
+  for (int a = 0; a < MAPS; ++a) {
+    m[a] = -INFINITY; l[a] = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) acc[a][c] = 0.f;
+  }
+  const int ncol = (dv + 63) / 64;
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+  for (int seg = kept > 0 ? 0 : 1; seg < 2; ++seg) {
+    const int j_lo = seg == 0 ? 0 : lo, j_hi = seg == 0 ? kept - 1 : pos;
+    for (int j0 = j_lo; j0 <= j_hi; j0 += 64) {
+      const int j = j0 + lane;
+      int blk = -1;
+      if (j <= j_hi) blk = table[j / kParBlock];
+      const bool valid = blk >= 0 && blk < num_blocks;
+      float s[MAPS], p[MAPS];
+      bool any = false;
+#pragma unroll
+      for (int a = 0; a < MAPS; ++a) {
+        s[a] = -INFINITY;
+        if (valid) {
+          const T* krow = kcache + (((long)blk * G + g) * kParBlock + (j % kParBlock)) * k_row + a * d;
+          float dot = dot_row(qs[wave] + a * d, krow, d, vec != 0);
+          if (softcap > 0.f) dot = softcap * tanhf(dot * inv_cap);
+          s[a] = dot;
+        }
+        const float m_new = fmaxf(m[a], wave_max(s[a]));
+        if (m_new == -INFINITY) { p[a] = 0.f; continue; }      // (uniform over the wave)
+        p[a] = valid ? expf(s[a] - m_new) : 0.f;
+        const float corr = (m[a] == -INFINITY) ? 0.f : expf(m[a] - m_new);
+        l[a] = l[a] * corr + wave_sum(p[a]);
+        m[a] = m_new;
+#pragma unroll
+        for (int c = 0; c < kMultiMaxDV / 64; ++c) acc[a][c] *= corr;
+        any = true;
+      }
+      if (!any) continue;
+      const int nk = (j_hi - j0 + 1) < 64 ? (j_hi - j0 + 1) : 64;
+      for (int jj = 0; jj < nk; ++jj) {
+        float pj[MAPS];
+        bool zero = true;
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a) { pj[a] = __shfl(p[a], jj, 64); zero = zero && pj[a] == 0.f; }
+        const int bj = __shfl(blk, jj, 64);
+        if (zero) continue;                       // (uniform: an unreadable key, or weights that underflowed)
+        const T* vrow = vcache + (((long)bj * G + g) * kParBlock + ((j0 + jj) % kParBlock)) * v_row + v_off;
+#pragma unroll
+        for (int c = 0; c < kMultiMaxDV / 64; ++c)
+          if (c < ncol) {
+            const int col = c * 64 + lane;
+            if (col < dv) {
+              const float v = (float)vrow[col];
+#pragma unroll
+              for (int a = 0; a < MAPS; ++a) acc[a][c] += pj[a] * v;
+            }
+          }
+      }
+    }
+  }
+  float o[kMultiMaxDV / 64];
+  const float i0 = l[0] > 0.f ? 1.f / l[0] : 0.f;
+  if constexpr (MAPS == 1) {
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) o[c] = acc[0][c] * i0;
+  } else {
+    // the two maps combined, normalised over the head's values, and gated
+    const float i1 = l[1] > 0.f ? 1.f / l[1] : 0.f;
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) {
+      o[c] = 0.f;
+      if (c < ncol && c * 64 + lane < dv) { o[c] = acc[0][c] * i0 - lam * acc[1][c] * i1; ss += o[c] * o[c]; }
+    }
+    ss = wave_sum(ss);
+    const float r = post / sqrtf(ss / dv + eps);
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) o[c] *= r;
+  }
+#pragma unroll
+  for (int c = 0; c < kMultiMaxDV / 64; ++c)
+    if (c < ncol) {
+      const int col = c * 64 + lane;
+      if (col < dv) {
+        float v = o[c];
+        if (gate) v *= 1.f / (1.f + expf(-gate[(long)t * ldg + (long)h * dv + col]));
+        orow[col] = (OT)v;
+      }
+    }
+}
+
+// ---- real-gated linear recurrence ----------------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh32(float x) {
+  const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
+  return 0.5f * x * (1.f + tanhf(u));
+}
+
+// One token of one channel: (decay a, input b) of S <- a S + b.
+__device__ __forceinline__ void rglru_terms(float u, float gr, float gi, float cl, float& a, float& b) {
+  const float r = 1.f / (1.f + expf(-gr)), i = 1.f / (1.f + expf(-gi));
+  const float la = -cl * r;
+  a = expf(la);
+  b = sqrtf(-expm1f(2.f * la)) * i * u;
+}
+
+// grid (sequences, channel blocks of 64), SEGS waves per workgroup: wave s scans the s-th stretch of the step's tokens for
+// 64 channels. First pass: every stretch from zero, keeping only its (decay product, end value); the stretches are joined
+// in order; second pass: every stretch again from its true start, writing the read-outs. A step with few tokens per
+// sequence runs with one stretch and one pass.
+template <typename OT, int SEGS>
+__global__ __launch_bounds__(64 * SEGS) void rglru_scan_kernel(
+    OT* __restrict__ out, long ldo, const float* __restrict__ u, long ldu, const float* __restrict__ gates, long ldg,
+    const float* __restrict__ ypre, long ldy, const float* __restrict__ clam, float* __restrict__ state,
+    const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots, int W, int bw, int state_rows) {
+  __shared__ float seg_a[SEGS][64], seg_b[SEGS][64];
+  const int b = blockIdx.x;
+  const int t0 = q_start[b], n = q_start[b + 1] - t0, c0 = ctx[b], slot = slots[b];
+  if (n <= 0 || slot < 0 || slot >= state_rows) return;              // (whole workgroup)
+  const int lane = threadIdx.x & 63, sg = SEGS == 1 ? 0 : (int)(threadIdx.x >> 6);
+  const int c = blockIdx.y * 64 + lane;
+  const bool on = c < W;
+  const int cc = on ? c : 0;
+  const int gcol = (cc / bw) * 2 * bw + cc % bw;
+  const float cl = clam[cc];
+  const int per = (n + SEGS - 1) / SEGS;
+  const int r0 = min(n, sg * per), r1 = min(n, r0 + per);
+  float S = 0.f;
+  if constexpr (SEGS > 1) {
+    float A = 1.f, Bv = 0.f;
+    for (int r = r0; r < r1; ++r) {
+      const long t = t0 + r;
+      float a, bb;
+      rglru_terms(u[t * ldu + cc], gates[t * ldg + gcol], gates[t * ldg + gcol + bw], cl, a, bb);
+      A *= a; Bv = a * Bv + bb;
+    }
+    seg_a[sg][lane] = A; seg_b[sg][lane] = Bv;
+    __syncthreads();
+    S = c0 > 0 ? state[(long)slot * W + cc] : 0.f;
+    for (int k = 0; k < sg; ++k) S = seg_a[k][lane] * S + seg_b[k][lane];
+  } else {
+    S = c0 > 0 ? state[(long)slot * W + cc] : 0.f;
+  }
+  for (int r = r0; r < r1; ++r) {
+    const long t = t0 + r;
+    float a, bb;
+    rglru_terms(u[t * ldu + cc], gates[t * ldg + gcol], gates[t * ldg + gcol + bw], cl, a, bb);
+    S = a * S + bb;
+    if (on) out[t * ldo + c] = (OT)(S * gelu_tanh32(ypre[t * ldy + c]));
+  }
+  // (a short step may leave the last stretches empty: the one that holds the step's last token has the end state)
+  if (on && r1 == n && r1 > r0) state[(long)slot * W + c] = S;
+}
+
+// ---- activation, scaling ---------------------------------------------------------------------------------------------
+template <typename OT>
+__global__ __launch_bounds__(256) void xielu_kernel(OT* __restrict__ act, const float* __restrict__ z, int M, int F, long ldz,
+                                                    long lda, const float* __restrict__ pq) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long)M * F) return;
+  const int m = (int)(i / F), c = (int)(i % F);
+  const float ap = pq[0], aq = pq[1];          // softplus(p), 1/2 + softplus(q)
+  const float v = z[(long)m * ldz + c];
+  const float r = v > 0.f ? ap * v * v + 0.5f * v : aq * (expm1f(v) - v) + 0.5f * v;
+  act[(long)m * lda + c] = (OT)r;
+}
+
+__global__ __launch_bounds__(256) void scale_rows_kernel(float* __restrict__ x, int M, int N, long ld, float s) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long)M * N) return;
+  x[(i / N) * ld + i % N] *= s;
+}
+
+}  // namespace dlia
+
+using namespace dlia;
+
+extern "C" void dlia_par_norm(void* out, int out_f32, float* out32, float* x, const float* ya, const float* yb, const float* ls1,
+                              const float* ls2, const float* w, float* carry, const int* tok_seq, int T, int state_rows, int H,
+                              long ldx, long ldya, long ldyb, long ldo, float eps, hipStream_t stream) {
+  if (T <= 0) return;
+  if (out_f32 || !out)
+    hipLaunchKernelGGL(par_norm_kernel<float>, dim3(T), dim3(kParThreads), 0, stream, (float*)out, out32, x, ya, yb, ls1, ls2, w,
+                       carry, tok_seq, T, state_rows, H, ldx, ldya, ldyb, ldo, eps);
+  else
+    hipLaunchKernelGGL(par_norm_kernel<bf16>, dim3(T), dim3(kParThreads), 0, stream, (bf16*)out, out32, x, ya, yb, ls1, ls2, w,
+                       carry, tok_seq, T, state_rows, H, ldx, ldya, ldyb, ldo, eps);
+}
+
+extern "C" void dlia_token_shift(void* out, int out_f32, const float* n32, const float* carry, const float* mu, const int* tok_pos,
+                                 const int* tok_seq, int T, int state_rows, int H, long ldo, hipStream_t stream) {
+  if (T <= 0) return;
+  if (out_f32)
+    hipLaunchKernelGGL(token_shift_kernel<float>, dim3(T), dim3(kParThreads), 0, stream, (float*)out, n32, carry, mu, tok_pos,
+                       tok_seq, state_rows, H, ldo);
+  else
+    hipLaunchKernelGGL(token_shift_kernel<bf16>, dim3(T), dim3(kParThreads), 0, stream, (bf16*)out, n32, carry, mu, tok_pos,
+                       tok_seq, state_rows, H, ldo);
+}
+
+extern "C" void dlia_rope_cache_write(float* q, long ldq, int q_vecs, int q_stride, int q_off, void* q_out, long ldqo, int q_cols,
+                                      float* kv, long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols,
+                                      void* kcache, void* vcache, int f32, int G, int dims, int interleaved, const float* cos_t,
+                                      const float* sin_t, int table_pos, const int* tok_pos, const int* tok_seq,
+                                      const int* block_table, int T, int max_blocks, int num_blocks, int table_rows,
+                                      hipStream_t stream) {
+  if (T <= 0) return;
+  if (f32)
+    hipLaunchKernelGGL(rope_cache_write_kernel<float>, dim3(T), dim3(kParThreads), 0, stream, q, ldq, q_vecs, q_stride, q_off,
+                       (float*)q_out, ldqo, q_cols, kv, ldkv, k_cols, k_vecs, k_stride, k_off, v_cols, (float*)kcache,
+                       (float*)vcache, G, dims, interleaved, cos_t, sin_t, table_pos, tok_pos, tok_seq, block_table, max_blocks,
+                       num_blocks, table_rows);
+  else
+    hipLaunchKernelGGL(rope_cache_write_kernel<bf16>, dim3(T), dim3(kParThreads), 0, stream, q, ldq, q_vecs, q_stride, q_off,
+                       (bf16*)q_out, ldqo, q_cols, kv, ldkv, k_cols, k_vecs, k_stride, k_off, v_cols, (bf16*)kcache,
+                       (bf16*)vcache, G, dims, interleaved, cos_t, sin_t, table_pos, tok_pos, tok_seq, block_table, max_blocks,
+                       num_blocks, table_rows);
+}
+
+template <typename T, typename OT>
+static void launch_multi(int maps, dim3 grid, hipStream_t stream, void* out, long ldo, const float* q, long ldq, int q_head,
+                         const void* kc, int k_row, const void* vc, int v_row, int v_off, const int* tok_pos, const int* tok_seq,
+                         const int* table, int items, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
+                         float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
+                         const float* gate, long ldg, int vec) {
+  if (maps == 2)
+    hipLaunchKernelGGL((multi_attention_kernel<T, OT, 2>), grid, dim3(256), 0, stream, (OT*)out, ldo, q, ldq, q_head, (const T*)kc,
+                       k_row, (const T*)vc, v_row, v_off, tok_pos, tok_seq, table, items, max_blocks, num_blocks, table_rows, H, G,
+                       d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, vec);
+  else
+    hipLaunchKernelGGL((multi_attention_kernel<T, OT, 1>), grid, dim3(256), 0, stream, (OT*)out, ldo, q, ldq, q_head, (const T*)kc,
+                       k_row, (const T*)vc, v_row, v_off, tok_pos, tok_seq, table, items, max_blocks, num_blocks, table_rows, H, G,
+                       d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, vec);
+}
+
+extern "C" void dlia_multi_attention(void* out, long ldo, const float* q, long ldq, int q_head, const void* kcache, int k_row,
+                                     const void* vcache, int v_row, int v_off, int f32, const int* tok_pos, const int* tok_seq,
+                                     const int* block_table, int T, int max_blocks, int num_blocks, int table_rows, int H, int G,
+                                     int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam,
+                                     float post, float eps, const float* gate, long ldg, hipStream_t stream) {
+  const int items = T * H;
+  if (items <= 0) return;
+  const dim3 grid((items + 3) / 4);
+  const int per = f32 ? 4 : 8;
+  const int vec = d % per == 0 && k_row % per == 0 && (uintptr_t)kcache % 16 == 0;
+  if (f32)
+    launch_multi<float, float>(maps, grid, stream, out, ldo, q, ldq, q_head, kcache, k_row, vcache, v_row, v_off, tok_pos, tok_seq,
+                               block_table, items, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first,
+                               softcap, lam, post, eps, gate, ldg, vec);
+  else
+    launch_multi<bf16, bf16>(maps, grid, stream, out, ldo, q, ldq, q_head, kcache, k_row, vcache, v_row, v_off, tok_pos, tok_seq,
+                             block_table, items, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first,
+                             softcap, lam, post, eps, gate, ldg, vec);
+}
+
+extern "C" void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg,
+                                const float* ypre, long ldy, const float* clam, float* state, const int* q_start, const int* ctx,
+                                const int* slots, int B, int max_q, int W, int bw, int state_rows, hipStream_t stream) {
+  if (B <= 0 || max_q <= 0) return;
+  const dim3 grid(B, (W + 63) / 64);
+#define DLIA_RGLRU(OT, SEGS)                                                                                              \
+  hipLaunchKernelGGL((rglru_scan_kernel<OT, SEGS>), grid, dim3(64 * SEGS), 0, stream, (OT*)out, ldo, u, ldu, gates, ldg, ypre, \
+                     ldy, clam, state, q_start, ctx, slots, W, bw, state_rows)
+  if (max_q >= 256) {
+    if (out_f32) DLIA_RGLRU(float, 16); else DLIA_RGLRU(bf16, 16);
+  } else if (max_q >= 16) {
+    if (out_f32) DLIA_RGLRU(float, 4); else DLIA_RGLRU(bf16, 4);
+  } else {
+    if (out_f32) DLIA_RGLRU(float, 1); else DLIA_RGLRU(bf16, 1);
+  }
+#undef DLIA_RGLRU
+}
+
+extern "C" void dlia_xielu(void* act, int out_f32, const float* z, int M, int F, long ldz, long lda, const float* pq,
+                           hipStream_t stream) {
+  const long n = (long)M * F;
+  if (n <= 0) return;
+  const dim3 grid((unsigned)((n + 255) / 256));
+  if (out_f32) hipLaunchKernelGGL(xielu_kernel<float>, grid, dim3(256), 0, stream, (float*)act, z, M, F, ldz, lda, pq);
+  else hipLaunchKernelGGL(xielu_kernel<bf16>, grid, dim3(256), 0, stream, (bf16*)act, z, M, F, ldz, lda, pq);
+}
+
+extern "C" void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStream_t stream) {
+  const long n = (long)M * N;
+  if (n <= 0) return;
+  hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, M, N, ld, s);
+}
