@@ -1,0 +1,255 @@
+"""Every mechanism of the Tezesun design alone: the package's torch operations (CPU) and its HIP kernels (`gpu` marker)
+against the plain float64 functions of `tezesun_oracle`, on small inputs made here."""
+import math
+
+import pytest
+import torch
+
+import tezesun_oracle as O
+
+F64 = torch.float64
+
+
+def rnd(*shape, seed=0, std=1.0):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=F64) * std
+
+
+def close(got, ref, tol=2e-5):
+    ref = ref.to(F64)
+    err = (got.detach().cpu().to(F64) - ref).abs().max().item() / max(1.0, ref.abs().max().item())
+    assert err < tol, err
+
+
+# ---- torch operations (the CPU executor's) ---------------------------------------------------------------------------
+def test_xielu_and_token_shift():
+    from distributed_llm_inference_amd.ops import reference as R
+    z = rnd(7, 33, seed=1, std=3.0)
+    for p, q in [(0.3, -0.7), (-2.0, 1.5), (0.0, 0.0)]:
+        close(R.xielu(z.float(), torch.tensor(p), torch.tensor(q)), O.xielu(z, torch.tensor(p, dtype=F64), torch.tensor(q, dtype=F64)))
+    h, mu = rnd(9, 20, seed=2), torch.rand(20, dtype=F64)
+    ref = O.token_shift(h, mu)
+    a, last = R.token_shift(h[:4].float(), torch.zeros(20), mu.float())           # in two portions: the last row is carried
+    b, _ = R.token_shift(h[4:].float(), last, mu.float())
+    close(torch.cat([a, b]), ref)
+
+
+@pytest.mark.parametrize("interleaved", [True, False])
+@pytest.mark.parametrize("dims,D", [(8, 8), (4, 10), (2, 2)])
+def test_partial_rotation_and_scaled_frequencies(interleaved, dims, D):
+    from distributed_llm_inference_amd.models.rope import rope_table
+    from distributed_llm_inference_amd.models.spec import RopeScaling
+    from distributed_llm_inference_amd.ops import reference as R
+    for sc in (None, {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}, {"factor": 8.0, "original": 1000, "fast": 32.0, "slow": 1.0}):
+        rot = {"dims": dims, "base": 100.0, **({"scaling": sc} if sc else {})}
+        rs = RopeScaling(factor=sc["factor"], rope_type="yarn", beta_fast=sc["fast"], beta_slow=sc["slow"],
+                         original_max_position_embeddings=sc["original"]) if sc else None
+        cos, sin = rope_table(dims, 100.0, rs, 50)
+        rc, rsn = O.rope_angles(rot, 50)
+        close(cos, rc, 1e-6)
+        close(sin, rsn, 1e-6)
+        x = rnd(50, 3, D, seed=3)
+        got = R.rope_partial(x.float(), cos, sin, torch.arange(50), interleaved)
+        close(got, O.rotate(x, rc, rsn, interleaved))
+        # positions are the tokens' own, not their place in the step
+        got = R.rope_partial(x[:5].float(), cos, sin, torch.tensor([40, 41, 42, 43, 44]), interleaved)
+        close(got, O.rotate(x[:5], rc[40:45], rsn[40:45], interleaved))
+
+
+def _rglru_weights(W, nb, taps, H, seed):
+    bw = W // nb
+    return {"y": rnd(W, H, seed=seed, std=H ** -0.5), "y.b": rnd(W, seed=seed + 1, std=0.3), "x": rnd(W, H, seed=seed + 2, std=H ** -0.5),
+            "x.b": rnd(W, seed=seed + 3, std=0.3), "conv": rnd(W, taps, seed=seed + 4, std=0.6), "conv.b": rnd(W, seed=seed + 5, std=0.2),
+            "ra": rnd(nb, bw, bw, seed=seed + 6, std=bw ** -0.5), "ra.b": rnd(nb, bw, seed=seed + 7, std=0.5),
+            "ri": rnd(nb, bw, bw, seed=seed + 8, std=bw ** -0.5), "ri.b": rnd(nb, bw, seed=seed + 9, std=0.5),
+            "lam": rnd(W, seed=seed + 10, std=1.5) - 2.0, "o": torch.eye(W, dtype=F64)}
+
+
+@pytest.mark.parametrize("W,nb,taps", [(24, 3, 3), (16, 1, 1), (10, 10, 5)])
+def test_recurrent_unit_in_portions(W, nb, taps):
+    """conv -> block gates -> recurrence over several calls with the carried inputs and state, against the whole sequence."""
+    from distributed_llm_inference_amd.ops import reference as R
+    H, T = 12, 40
+    w, h = _rglru_weights(W, nb, taps, H, 20), rnd(T, H, seed=5)
+    ref = O.rglru(h, w)
+    carry, S, outs, t0 = torch.zeros(taps - 1, W), torch.zeros(W), [], 0
+    for n in (1, 2, 17, 1, 19):
+        hp = h[t0:t0 + n].float()
+        y = R.gelu_tanh(hp @ w["y"].float().T + w["y.b"].float())
+        u, carry = R.short_conv(hp @ w["x"].float().T + w["x.b"].float(), carry, w["conv"].float())
+        u = u + w["conv.b"].float()
+        gr, gi = torch.sigmoid(R.block_linear(u, w["ra"], w["ra.b"])), torch.sigmoid(R.block_linear(u, w["ri"], w["ri.b"]))
+        st, S = R.rglru_scan(u, gr, gi, w["lam"], S)
+        outs.append(st * y)
+        t0 += n
+    close(torch.cat(outs), ref, 5e-5)
+
+
+def test_attention_mask_with_kept_tokens_and_cap():
+    from distributed_llm_inference_amd.ops import reference as R
+    T, d, dv = 30, 6, 5
+    q, k, v = rnd(T, 2, d, seed=6), rnd(T, 1, d, seed=7), rnd(T, 1, dv, seed=8)
+    for window, keep, cap in [(4, 3, 2.0), (1, 0, 0.0), (7, 9, 0.5), (0, 0, 1.0)]:
+        ok = O.visible(T, window, keep)
+        ref = []
+        for hh in range(2):
+            s = (q[:, hh] @ k[:, 0].T) * 0.7
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            ref.append(torch.softmax(s.masked_fill(~ok, float("-inf")), -1) @ v[:, 0])
+        got = R.attention(q[10:].float(), k.float(), v.float(), 10, 0.7, window=window, keep_first=keep, softcap=cap)
+        close(got, torch.stack(ref, 1)[10:])
+
+
+# ---- HIP kernels ------------------------------------------------------------------------------------------------------
+def _K():
+    from distributed_llm_inference_amd import ops
+    return ops.load()
+
+
+def _meta(seqs, dev):
+    """seqs: [(slot, q_len, ctx)] -> tok_pos, tok_seq, q_start, ctx, slots (int32 on the device)."""
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=dev)
+    pos = [c + i for _, n, c in seqs for i in range(n)]
+    seq = [s for s, n, _ in seqs for _ in range(n)]
+    qs = [0]
+    for _, n, _ in seqs:
+        qs.append(qs[-1] + n)
+    return i32(pos), i32(seq), i32(qs), i32([c for _, _, c in seqs]), i32([s for s, _, _ in seqs])
+
+
+@pytest.mark.gpu
+def test_norm_residual_shift_and_carried_rows_hip():
+    """par_norm + token_shift over two steps of two sequences that sit in slots used before: positions 0 start from zeros,
+    portions go on from the slot's carried row."""
+    K, dev, H = _K(), "cuda", 40
+    x = rnd(12, H, seed=1)                      # sequence a: rows 0..6 (7 tokens), sequence b: rows 7..11 (5 tokens)
+    w, mu, ls1, ls2 = 1.0 + rnd(H, seed=2, std=0.1), torch.rand(H, dtype=F64), rnd(H, seed=3), rnd(H, seed=4)
+    ya, yb = rnd(12, H, seed=5), rnd(12, H, seed=6)
+    w2 = 1.0 + rnd(H, seed=7, std=0.1)
+    f = lambda t: t.float().to(dev).contiguous()
+    carry = torch.full((5, H), 7.0, device=dev)      # stale rows
+    got_s, got_n2 = {}, {}
+    for step, (ra, rb) in enumerate([((0, 3), (7, 9)), ((3, 7), (9, 12))]):
+        rows = list(range(*ra)) + list(range(*rb))
+        tok_pos, tok_seq, *_ = _meta([(3, ra[1] - ra[0], ra[0]), (1, rb[1] - rb[0], rb[0] - 7)], dev)
+        h = f(x[rows])
+        n32, xn, xs = torch.zeros(len(rows), H, device=dev), torch.zeros(len(rows), H, device=dev), torch.zeros(len(rows), H, device=dev)
+        K.par_norm(xn, n32, h, None, None, None, None, f(w), None, tok_seq, 1e-5)
+        K.token_shift(xs, n32, carry, f(mu), tok_pos, tok_seq)
+        K.par_norm(xn, n32, h, f(ya[rows]), f(yb[rows]), f(ls1), f(ls2), f(w2), carry, tok_seq, 1e-5)
+        for i, r in enumerate(rows):
+            got_s[r], got_n2[r] = xs[i].cpu(), xn[i].cpu()
+    for lo, hi in ((0, 7), (7, 12)):
+        n = O.rms(x[lo:hi], 1e-5) * w
+        ref_s = O.token_shift(n, mu)
+        ref_n2 = O.rms(x[lo:hi] + ls1 * ya[lo:hi] + ls2 * yb[lo:hi], 1e-5) * w2
+        close(torch.stack([got_s[r] for r in range(lo, hi)]), ref_s)
+        close(torch.stack([got_n2[r] for r in range(lo, hi)]), ref_n2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,G,d,dv,maps,window,keep,cap,dims,inter", [
+    (4, 2, 16, 24, 2, 40, 5, 10.0, 8, True), (2, 1, 8, 8, 1, 0, 0, 0.0, 8, False), (3, 3, 12, 70, 2, 3, 50, 0.0, 4, True),
+    (2, 2, 72, 130, 1, 33, 0, 3.0, 0, False), (6, 1, 10, 16, 2, 64, 1, 25.0, 10, True)])
+def test_rotation_cache_write_and_attention_hip(dtype, H, G, d, dv, maps, window, keep, cap, dims, inter):
+    """rope_cache_write + multi_attention over a paged cache whose blocks are in no order: a prompt portion, then another
+    that crosses block edges, then single tokens, against whole-sequence attention; two maps combined, normed and gated."""
+    K, dev = _K(), "cuda"
+    T, eps, lam, post, scale = 150, 1e-5, 0.37, 0.6, 0.3
+    q, k = rnd(T, H * maps, d, seed=1), rnd(T, G * maps, d, seed=2)
+    v, gate = rnd(T, G, dv, seed=3), rnd(T, H * dv, seed=4)
+    if dtype == torch.bfloat16:             # inputs that the cache holds exactly
+        k, v = k.bfloat16().to(F64), v.bfloat16().to(F64)
+    rot = {"dims": dims, "base": 50.0}
+    cos, sin = O.rope_angles(rot, T) if dims else (None, None)
+    qr, kr = (O.rotate(q, cos, sin, inter), O.rotate(k, cos, sin, inter)) if dims else (q, k)
+    ok = O.visible(T, window, keep)
+    heads = []
+    for hh in range(H):
+        g, per = hh // (H // G), []
+        for mp in range(maps):
+            s = (qr[:, maps * hh + mp] @ kr[:, maps * g + mp].T) * scale
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            per.append(torch.softmax(s.masked_fill(~ok, float("-inf")), -1) @ v[:, g])
+        heads.append(O.rms(per[0] - lam * per[1], eps) * post if maps == 2 else per[0])
+    ref = torch.cat(heads, -1) * (torch.sigmoid(gate) if maps == 2 else 1.0)
+    nblk = 9
+    kc = torch.zeros(nblk, G, 32, maps * d, device=dev, dtype=dtype)
+    vc = torch.zeros(nblk, G, 32, dv, device=dev, dtype=dtype)
+    table = torch.full((3, 6), -1, dtype=torch.int32, device=dev)
+    table[1, :5] = torch.tensor([7, 2, 5, 0, 3], dtype=torch.int32)
+    f = lambda t: t.float().to(dev).contiguous() if t is not None else None
+    z_all = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1)
+    qn, kn, vn = H * maps * d, G * maps * d, G * dv
+    got, t0 = [], 0
+    for n in (50, 47, 1, 1, 1, 50):
+        tok_pos, tok_seq, *_ = _meta([(1, n, t0)], dev)
+        z = f(z_all[t0:t0 + n])
+        out = torch.zeros(n, H * dv, device=dev, dtype=dtype)
+        K.rope_cache_write(z, H * maps, d, 0, None, 0, z[:, qn:], kn, G * maps, d, 0, vn, kc, vc, dims, inter, f(cos), f(sin), tok_pos, tok_seq, table)
+        K.multi_attention(out, z, maps * d, kc, vc, 0, tok_pos, tok_seq, table, H, d, dv, maps, scale, window, keep, cap, lam, post, eps,
+                          f(gate[t0:t0 + n]) if maps == 2 else None)
+        got.append(out.float().cpu())
+        t0 += n
+    close(torch.cat(got), ref, 2e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("W,nb,taps", [(24, 3, 3), (16, 1, 1), (100, 100, 4), (320, 4, 2)])
+def test_recurrent_unit_hip(W, nb, taps):
+    """short_conv_act + gemm_blocks + rglru_scan: two sequences in one step (a long portion that is scanned in segments
+    beside a single token), several steps, slots that held other values, against the whole sequences."""
+    K, dev, H = _K(), "cuda", 12
+    bw = W // nb
+    w = _rglru_weights(W, nb, taps, H, 30)
+    ha, hb = rnd(700, H, seed=8), rnd(40, H, seed=9)
+    ref_a, ref_b = O.rglru(ha, w), O.rglru(hb, w)
+    f = lambda t: t.float().to(dev).contiguous()
+    pre = lambda h: torch.cat([h @ w["y"].T + w["y.b"], h @ w["x"].T + w["x.b"]], 1)
+    za, zb = pre(ha), pre(hb)
+    wg, bg = f(torch.cat([w["ra"], w["ri"]], 1)), f(torch.cat([w["ra.b"], w["ri.b"]], 1).reshape(-1))
+    clam = f(8.0 * O.softplus(w["lam"]))
+    carry, state = torch.full((4, max(taps - 1, 1), W), 3.0, device=dev), torch.full((4, W), -2.0, device=dev)
+    got_a, got_b, a0, b0 = [], [], 0, 0
+    for na, nb_ in [(300, 1), (1, 1), (20, 2), (379, 36)]:
+        seqs = [(2, nb_, b0), (0, na, a0)]
+        _, _, q_start, ctx, slots = _meta(seqs, dev)
+        z = f(torch.cat([zb[b0:b0 + nb_], za[a0:a0 + na]]))
+        n = na + nb_
+        u, gates, out = torch.zeros(n, W, device=dev), torch.zeros(n, 2 * W, device=dev), torch.zeros(n, W, device=dev)
+        K.short_conv_act(u, z[:, W:], carry, f(w["conv"]), f(w["conv.b"]), q_start, ctx, slots, max(na, nb_), False)
+        K.gemm_blocks(gates, u, wg, bg, bw, 2 * bw)
+        K.rglru_scan(out, u, gates, z[:, :W], clam, state, q_start, ctx, slots, bw, max(na, nb_))
+        got_b.append(out[:nb_].cpu())
+        got_a.append(out[nb_:].cpu())
+        a0, b0 = a0 + na, b0 + nb_
+    close(torch.cat(got_a), ref_a, 5e-5)
+    close(torch.cat(got_b), ref_b, 5e-5)
+
+
+@pytest.mark.gpu
+def test_block_products_activation_and_scale_hip():
+    K, dev = _K(), "cuda"
+    x, w, b = rnd(37, 5 * 12, seed=1), rnd(5, 7, 12, seed=2), rnd(5, 7, seed=3)
+    ref = torch.einsum("tbi,boi->tbo", x.reshape(37, 5, 12), w) + b
+    out = torch.zeros(37, 5 * 7, device=dev)
+    K.gemm_blocks(out, x.float().to(dev), w.float().to(dev).contiguous(), b.float().to(dev).reshape(-1).contiguous(), 12, 7)
+    close(out, ref.reshape(37, -1))
+    # blocks that read overlapping-free slices of wider rows and write into wider rows (bf16 operands, fp32 sums)
+    xb, wb = rnd(20, 3 * 24, seed=4).bfloat16(), rnd(3, 10, 16, seed=5).bfloat16()
+    out = torch.zeros(20, 3 * 12, device=dev)
+    K.gemm_blocks(out, xb.to(dev), wb.to(dev).contiguous(), None, 24, 12)
+    ref = torch.einsum("tbi,boi->tbo", xb.to(F64).reshape(20, 3, 24)[:, :, :16], wb.to(F64))
+    close(out.reshape(20, 3, 12)[:, :, :10], ref, 1e-5)
+    z = rnd(9, 50, seed=6, std=3.0)
+    p, q = torch.tensor(0.4, dtype=F64), torch.tensor(-1.1, dtype=F64)
+    act = torch.zeros(9, 50, device=dev)
+    K.xielu(act, z.float().to(dev), torch.stack([O.softplus(p), 0.5 + O.softplus(q)]).float().to(dev))
+    close(act, O.xielu(z, p, q))
+    lg = rnd(4, 30, seed=7).float().to(dev)
+    ref = lg.cpu().to(F64).clone()
+    ref[:, :25] *= 1.7
+    K.scale_rows(lg, 25, 1.7)
+    close(lg, ref)
