@@ -141,6 +141,11 @@ class HybridGpuStage(GpuStage):
         self.runs = spec.layer_runs()
         if self.par:
             self.mfma_attn = [False] * len(self.specs)
+            # attention layers whose sizes are multiples of 8 run on the matrix cores in bf16 (values key-contiguous in the
+            # cache); other sizes, and the fp32 mode, on the one-wave-per-(token, head) kernel. DLIA_PAR_TILE_ATTN=0: all on that (A/B)
+            tile_ok = dtype == "bf16" and os.environ.get("DLIA_PAR_TILE_ATTN", "1") != "0"
+            self._tile = [tile_ok and ls.kind != "rglru" and self._score_dim(ls) % 8 == 0 and ls.maps * self._score_dim(ls) <= 1024
+                          for ls in self.specs]
             self._load_par(weights, f32, mat)
         elif self.gated:
             self._load_gated(weights, f32, mat)
@@ -297,7 +302,7 @@ class HybridGpuStage(GpuStage):
     def kv_block_bytes(self) -> int:
         e = 4 if self.act_dtype == torch.float32 else 2
         if self.par:
-            return max(1, sum(BLOCK * e * sum(self._par_rows(ls)) for ls in self.specs if ls.kind != "rglru"))
+            return max(1, sum(BLOCK * e * sum(self._par_rows(li)) for li, ls in enumerate(self.specs) if ls.kind != "rglru"))
         return max(1, sum(ls.kv_heads * BLOCK * (ls.dim + ls.vdim) * e for ls in self._attn_of_run if ls is not None))
 
     def _decode_state_bytes(self) -> int:
@@ -318,13 +323,18 @@ class HybridGpuStage(GpuStage):
             # attention: key rows hold a head's score maps side by side, value rows apart; latent attention: ONE row per token,
             # the normed latent followed by the rotated key part (the values are the row's first entries)
             self.kv = []
-            for ls in self.specs:
+            for li, ls in enumerate(self.specs):
                 if ls.kind == "rglru":
                     self.kv.append(None)
                     continue
-                kr, vr = self._par_rows(ls)
-                kc = torch.zeros(self.num_blocks, ls.kv_heads, BLOCK, kr // ls.kv_heads, device=dev, dtype=at)
-                self.kv.append((kc, torch.zeros(self.num_blocks, ls.kv_heads, BLOCK, vr // ls.kv_heads, device=dev, dtype=at) if vr else kc))
+                kr, vr = self._par_rows(li)
+                G = ls.kv_heads
+                kc = torch.zeros(self.num_blocks, G, BLOCK, kr // G, device=dev, dtype=at)
+                if self._tile[li]:        # values key-contiguous: [block][head][entry][32 tokens]
+                    vc = torch.zeros(self.num_blocks, G, vr // G, BLOCK, device=dev, dtype=at)
+                else:
+                    vc = torch.zeros(self.num_blocks, G, BLOCK, vr // G, device=dev, dtype=at) if vr else kc
+                self.kv.append((kc, vc))
             return
         # zero-filled: a row that was never written must hold finite values
         # (a layer on the MFMA attention kernels keeps K and V slabs of a block side by side, in fragment order)
@@ -636,10 +646,17 @@ class HybridGpuStage(GpuStage):
 
     # ---- stacks with parallel layers on one norm -----------------------------------------------------------------------
     @staticmethod
-    def _par_rows(ls) -> tuple:
-        """(entries of a token's key row, of its value row) in the cache of an attention layer, over all its key / value heads."""
+    def _score_dim(ls) -> int:
+        """Entries of one score map's keys."""
+        return ls.kv_rank + ls.rot_dim if ls.kind == "latent_attention" else ls.dim
+
+    def _par_rows(self, li: int) -> tuple:
+        """(entries of a token's key row, of its value row) in the cache of attention layer li, over all its key / value heads.
+        Latent attention keeps ONE row, the normed latent followed by the rotated key part; its values are the row's first
+        entries (the matrix-core kernel wants them key-contiguous as well: a second, transposed copy of the latent)."""
+        ls = self.specs[li]
         if ls.kind == "latent_attention":
-            return ls.kv_rank + ls.rot_dim, 0
+            return ls.kv_rank + ls.rot_dim, ls.kv_rank if self._tile[li] else 0
         return ls.kv_heads * ls.maps * ls.dim, ls.kv_heads * ls.vdim
 
     def _load_par(self, weights: StageWeights, f32, mat):
@@ -712,6 +729,8 @@ class HybridGpuStage(GpuStage):
                 cq, q32 = max(cq, ls.q_rank), max(q32, self._cols(p, "w_uq"))
                 q16, qa = max(q16, ls.heads * (ls.dim + ls.rot_dim)), max(qa, ls.heads * (ls.kv_rank + ls.rot_dim))
                 ol = max(ol, ls.heads * ls.kv_rank)
+            if ls.kind == "attention":
+                q16 = max(q16, ls.heads * ls.maps * ls.dim)
             if ls.ff:
                 z2, ac, yc = max(z2, self._cols(p, "w_up")), max(ac, ls.ff), max(yc, self._cols(p, "w_down"))
         ws_floats = self._ws_floats
@@ -723,7 +742,7 @@ class HybridGpuStage(GpuStage):
             h=torch.zeros(rows, H, device=dev), n32=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at),
             xs=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc), u=z(rows * uc), gates=z(rows * 2 * uc), mixed=z(rows * mc, at),
             ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2), act=z(rows * ac, at), cq=z(rows * cq, at), q32=z(rows * q32),
-            q16=z(rows * q16, at), qa=z(rows * qa), olat=z(rows * ol, at), ws=z(ws_floats + 4096),
+            q16=z(rows * q16, at), qa=z(rows * qa), qa16=z(rows * qa if any(self._tile) else 1, at), olat=z(rows * ol, at), ws=z(ws_floats + 4096),
             head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
 
     def _layers_par(self, wk, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int):
@@ -750,24 +769,39 @@ class HybridGpuStage(GpuStage):
                 qn, kn, vn = Hh * M * d, G * M * d, G * dv
                 kc, vc = self.kv[li]
                 mixed = view(wk.mixed, Hh * dv)
-                K.rope_cache_write(z, Hh * M, d, 0, None, 0, z[:, qn:], kn, G * M, d, 0, vn, kc, vc, ls.rope_dims, ls.rope_interleaved,
-                                   p["cos"], p["sin"], tok_pos, tok_seq, table)
-                K.multi_attention(mixed, z, M * d, kc, vc, 0, tok_pos, tok_seq, table, Hh, d, dv, M, ls.scale, ls.window or 0,
-                                  ls.keep_first, ls.softcap, p["lam"], 1.0 - ls.diff, eps,
-                                  z[:, qn + kn + vn:qn + kn + vn + Hh * dv] if ls.out_gate else None)
+                gate = z[:, qn + kn + vn:qn + kn + vn + Hh * dv] if ls.out_gate else None
+                post = 1.0 - ls.diff if M == 2 else 1.0
+                if self._tile[li]:
+                    q16 = view(wk.q16, qn)
+                    K.rope_cache_write(z, Hh * M, d, 0, q16, qn, z[:, qn:], kn, G * M, d, 0, kn, vn, True, kc, vc, ls.rope_dims,
+                                       ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
+                    K.tile_attention(mixed, q16, M * d, kc, vc, q_start, ctx, slots, table, max_q, Hh, d, dv, M, ls.scale, ls.window or 0,
+                                     ls.keep_first, ls.softcap, p["lam"], post, eps, gate)
+                else:
+                    K.rope_cache_write(z, Hh * M, d, 0, None, 0, z[:, qn:], kn, G * M, d, 0, kn, vn, False, kc, vc, ls.rope_dims,
+                                       ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
+                    K.multi_attention(mixed, z, M * d, kc, vc, 0, tok_pos, tok_seq, table, Hh, d, dv, M, ls.scale, ls.window or 0,
+                                      ls.keep_first, ls.softcap, p["lam"], post, eps, gate)
             else:
                 Hh, d, dr, dv, R, qr = ls.heads, ls.dim, ls.rot_dim, ls.vdim, ls.kv_rank, ls.q_rank
-                kc = self.kv[li][0]
+                kc, vc = self.kv[li]
                 cq, q32 = view(wk.cq, qr), view(wk.q32, self._cols(p, "w_uq"))
                 q16, qa, olat, mixed = view(wk.q16, Hh * (d + dr)), view(wk.qa, Hh * (R + dr)), view(wk.olat, Hh * R), view(wk.mixed, Hh * dv)
                 K.norm32(cq, z[:, :qr], None, None, p["dq_norm"], None, eps, 0.0)
                 K.norm32(z[:, qr:qr + R], z[:, qr:qr + R], None, None, p["dkv_norm"], None, eps, 0.0)       # (in place)
                 self._mm(wk, q32, cq, p, "w_uq")
-                K.rope_cache_write(q32, Hh, d + dr, d, q16, Hh * (d + dr), z[:, qr:], R + dr, 1, R + dr, R, 0, kc, None, ls.rope_dims,
-                                   ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
-                K.gemm_blocks(qa, q16, p["w_abs"], None, d + dr, R + dr)
-                K.multi_attention(olat, qa, R + dr, kc, kc, 0, tok_pos, tok_seq, table, Hh, R + dr, R, 1, ls.scale, 0, 0, 0.0, 0.0, 1.0,
-                                  eps, None)
+                tile = self._tile[li]
+                K.rope_cache_write(q32, Hh, d + dr, d, q16, Hh * (d + dr), z[:, qr:], R + dr, 1, R + dr, R, 0, R if tile else 0, tile, kc,
+                                   vc if tile else None, ls.rope_dims, ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
+                if tile:
+                    qa16 = view(wk.qa16, Hh * (R + dr))
+                    K.gemm_blocks(qa16, q16, p["w_abs"], None, d + dr, R + dr)
+                    K.tile_attention(olat, qa16, R + dr, kc, vc, q_start, ctx, slots, table, max_q, Hh, R + dr, R, 1, ls.scale, 0, 0, 0.0,
+                                     0.0, 1.0, eps, None)
+                else:
+                    K.gemm_blocks(qa, q16, p["w_abs"], None, d + dr, R + dr)
+                    K.multi_attention(olat, qa, R + dr, kc, kc, 0, tok_pos, tok_seq, table, Hh, R + dr, R, 1, ls.scale, 0, 0, 0.0, 0.0, 1.0,
+                                      eps, None)
                 K.gemm_blocks(mixed, olat, p["w_uv"], None, R, dv)
             ya, yb = view(wk.ya, self._cols(p, "w_o")), None
             self._mm(wk, ya, mixed, p, "w_o")

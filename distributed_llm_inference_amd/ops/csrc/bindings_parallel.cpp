@@ -97,8 +97,8 @@ void token_shift(Tensor out, const Tensor& n32, const Tensor& carry, const Tenso
 // q [T, >= q_cols] fp32 (rotated in place: q_vecs vectors `q_stride` apart, entries [q_off, q_off + dims) of each); kv [T, k_cols + v_cols]
 // fp32 (k rotated in place the same way, then k and v rows written to the caches [blocks, G, 32, k_cols / G] and [blocks, G, 32, v_cols / G]).
 void rope_cache_write(Tensor q, int64_t q_vecs, int64_t q_stride, int64_t q_off, const std::optional<Tensor>& q_out, int64_t q_cols,
-                      Tensor kv, int64_t k_cols, int64_t k_vecs, int64_t k_stride, int64_t k_off, int64_t v_cols, Tensor kcache,
-                      const std::optional<Tensor>& vcache, int64_t dims, bool interleaved, OptTensor cos_t, OptTensor sin_t,
+                      Tensor kv, int64_t k_cols, int64_t k_vecs, int64_t k_stride, int64_t k_off, int64_t v_src, int64_t v_cols,
+                      bool v_t, Tensor kcache, const std::optional<Tensor>& vcache, int64_t dims, bool interleaved, OptTensor cos_t, OptTensor sin_t,
                       const Tensor& tok_pos, const Tensor& tok_seq, const Tensor& block_table) {
   DLIA_ON_DEVICE_OF(kcache);
   check_fmat(q, "q"); check_fmat(kv, "kv"); check_act(kcache, "kcache");
@@ -108,7 +108,7 @@ void rope_cache_write(Tensor q, int64_t q_vecs, int64_t q_stride, int64_t q_off,
   DLIA_CHECK(dims >= 0 && dims % 2 == 0 && q_vecs >= 0 && k_vecs >= 0 && q_stride >= 1 && k_stride >= 1, "rope_cache_write: rotation geometry");
   DLIA_CHECK(q_cols <= q.size(1) && (q_vecs == 0 || (q_vecs - 1) * q_stride + q_off + dims <= q.size(1)) && q_off >= 0,
              "rope_cache_write: rotated q entries beyond the row");
-  DLIA_CHECK(k_cols >= 1 && v_cols >= 0 && k_cols + v_cols <= kv.size(1) && k_off >= 0 &&
+  DLIA_CHECK(k_cols >= 1 && v_cols >= 0 && k_cols <= kv.size(1) && v_src >= 0 && v_src + v_cols <= kv.size(1) && k_off >= 0 &&
              (k_vecs == 0 || (k_vecs - 1) * k_stride + k_off + dims <= k_cols), "rope_cache_write: rotated k entries beyond the row");
   DLIA_CHECK(kcache.dim() == 4 && kcache.is_contiguous() && kcache.size(2) == 32, "rope_cache_write: kcache [blocks, G, 32, dk]");
   const int64_t G = kcache.size(1);
@@ -117,8 +117,8 @@ void rope_cache_write(Tensor q, int64_t q_vecs, int64_t q_stride, int64_t q_off,
   if (vcache.has_value()) {
     check_act(*vcache, "vcache");
     DLIA_CHECK(vcache->dim() == 4 && vcache->is_contiguous() && vcache->size(0) == kcache.size(0) && vcache->size(1) == G &&
-               vcache->size(2) == 32 && G * vcache->size(3) == v_cols && vcache->scalar_type() == kcache.scalar_type(),
-               "rope_cache_write: vcache [blocks, G, 32, dv] of the k cache's type");
+               vcache->size(v_t ? 3 : 2) == 32 && G * vcache->size(v_t ? 2 : 3) == v_cols && vcache->scalar_type() == kcache.scalar_type(),
+               "rope_cache_write: vcache [blocks, G, 32, dv] (or [blocks, G, dv, 32]) of the k cache's type");
     vp = vcache->data_ptr();
   } else {
     DLIA_CHECK(v_cols == 0, "rope_cache_write: values without a cache");
@@ -137,8 +137,8 @@ void rope_cache_write(Tensor q, int64_t q_vecs, int64_t q_stride, int64_t q_off,
     cp = cos_t->data_ptr<float>(); sp = sin_t->data_ptr<float>(); table_pos = (int)cos_t->size(0);
   }
   dlia_rope_cache_write(q.data_ptr<float>(), q.stride(0), (int)q_vecs, (int)q_stride, (int)q_off, qo, ldqo, (int)q_cols,
-                        kv.data_ptr<float>(), kv.stride(0), (int)k_cols, (int)k_vecs, (int)k_stride, (int)k_off, (int)v_cols,
-                        kcache.data_ptr(), vp, is_f32(kcache), (int)G, (int)dims, interleaved ? 1 : 0, cp, sp, table_pos,
+                        kv.data_ptr<float>(), kv.stride(0), (int)k_cols, (int)k_vecs, (int)k_stride, (int)k_off, (int)v_src, (int)v_cols,
+                        v_t ? 1 : 0, kcache.data_ptr(), vp, is_f32(kcache), (int)G, (int)dims, interleaved ? 1 : 0, cp, sp, table_pos,
                         tok_pos.data_ptr<int>(), tok_seq.data_ptr<int>(), block_table.data_ptr<int>(), (int)T, (int)block_table.size(1),
                         (int)kcache.size(0), (int)block_table.size(0), cur_stream());
 }
@@ -173,6 +173,40 @@ void multi_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& 
                        block_table.data_ptr<int>(), (int)T, (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0),
                        (int)H, (int)G, (int)d, (int)dv, (int)maps, (float)scale, (int)window, (int)keep_first, (float)softcap,
                        (float)lam, (float)post, (float)eps, gp, ldg, cur_stream());
+}
+
+// The same attention on the matrix cores: bf16, q [T, .] bf16, values key-contiguous in vt [blocks, G, dv, 32]; per sequence
+// (q_start, ctx, slots) in tiles of 16 tokens.
+void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& kcache, const Tensor& vt, const Tensor& q_start,
+                    const Tensor& ctx, const Tensor& slots, const Tensor& block_table, int64_t max_q, int64_t H, int64_t d, int64_t dv,
+                    int64_t maps, double scale, int64_t window, int64_t keep_first, double softcap, double lam, double post, double eps,
+                    OptTensor gate) {
+  DLIA_ON_DEVICE_OF(out);
+  check_mat(out, "out"); check_mat(q, "q");
+  check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots"); check_i32(block_table, "block_table");
+  DLIA_CHECK(out.is_cuda() && q.is_cuda() && kcache.is_cuda() && vt.is_cuda() && out.scalar_type() == at::kBFloat16 &&
+             q.scalar_type() == at::kBFloat16 && kcache.scalar_type() == at::kBFloat16 && vt.scalar_type() == at::kBFloat16,
+             "tile_attention: bfloat16 on the GPU");
+  const int64_t T = out.size(0), B = ctx.numel();
+  DLIA_CHECK(kcache.dim() == 4 && vt.dim() == 4 && kcache.is_contiguous() && vt.is_contiguous() && kcache.size(2) == 32 && vt.size(3) == 32 &&
+             kcache.size(0) == vt.size(0) && kcache.size(1) == vt.size(1) && vt.size(2) == dv, "tile_attention: kcache [blocks, G, 32, row], vt [blocks, G, dv, 32]");
+  const int64_t G = kcache.size(1), k_row = kcache.size(3);
+  DLIA_CHECK((maps == 1 || maps == 2) && d >= 8 && maps * d <= k_row && H >= 1 && H % G == 0 && out.size(1) == H * dv && q.size(0) >= T &&
+             q_head >= maps * d && (H - 1) * q_head + maps * d <= q.size(1), "tile_attention: head geometry");
+  DLIA_CHECK(q_start.numel() >= B + 1 && slots.numel() >= B && block_table.dim() == 2 && max_q >= 0 && max_q <= T && window >= 0 && keep_first >= 0,
+             "tile_attention: metadata");
+  const float* gp = nullptr; long ldg = 0;
+  if (gate.has_value()) {
+    check_fmat(*gate, "gate");
+    DLIA_CHECK(gate->size(0) >= T && gate->size(1) == H * dv, "tile_attention: gate [T, H * dv]");
+    gp = gate->data_ptr<float>(); ldg = gate->stride(0);
+  }
+  const int rc = dlia_tile_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), (int)q_head, kcache.data_ptr(), (int)k_row,
+                                     vt.data_ptr(), q_start.data_ptr<int>(), ctx.data_ptr<int>(), slots.data_ptr<int>(), block_table.data_ptr<int>(),
+                                     (int)B, (int)max_q, (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0), (int)H, (int)G,
+                                     (int)d, (int)dv, (int)maps, (float)scale, (int)window, (int)keep_first, (float)softcap, (float)lam,
+                                     (float)post, (float)eps, gp, ldg, cur_stream());
+  DLIA_CHECK(rc == 0, "tile_attention: sizes must be multiples of 8 (d, key row, q head stride, q row), maps * d <= 1024, dv <= 512");
 }
 
 // out [T, W] = S_t * gelu_tanh(ypre); u [T, W] conv output, gates [T, blocks * 2 bw] (per block: the decay gate's bw logits, then
@@ -224,8 +258,9 @@ void gemm_blocks(Tensor out, const Tensor& x, const Tensor& w, OptTensor bias, i
 TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("par_norm(Tensor(a!)? out, Tensor(b!) out32, Tensor(c!) x, Tensor? ya, Tensor? yb, Tensor? ls1, Tensor? ls2, Tensor? w, Tensor(d!)? carry, Tensor tok_seq, float eps) -> ()");
   m.def("token_shift(Tensor(a!) out, Tensor n32, Tensor carry, Tensor mu, Tensor tok_pos, Tensor tok_seq) -> ()");
-  m.def("rope_cache_write(Tensor(a!) q, int q_vecs, int q_stride, int q_off, Tensor(b!)? q_out, int q_cols, Tensor(c!) kv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols, Tensor(d!) kcache, Tensor(e!)? vcache, int dims, bool interleaved, Tensor? cos_t, Tensor? sin_t, Tensor tok_pos, Tensor tok_seq, Tensor block_table) -> ()");
+  m.def("rope_cache_write(Tensor(a!) q, int q_vecs, int q_stride, int q_off, Tensor(b!)? q_out, int q_cols, Tensor(c!) kv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols, bool v_t, Tensor(d!) kcache, Tensor(e!)? vcache, int dims, bool interleaved, Tensor? cos_t, Tensor? sin_t, Tensor tok_pos, Tensor tok_seq, Tensor block_table) -> ()");
   m.def("multi_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vcache, int v_off, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate) -> ()");
+  m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate) -> ()");
   m.def("rglru_scan(Tensor(a!) out, Tensor u, Tensor gates, Tensor ypre, Tensor clam, Tensor(b!) state, Tensor q_start, Tensor ctx, Tensor slots, int bw, int max_q) -> ()");
   m.def("xielu(Tensor(a!) act, Tensor z, Tensor pq) -> ()");
   m.def("scale_rows(Tensor(a!) x, int cols, float s) -> ()");
@@ -237,6 +272,7 @@ TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
   m.impl("token_shift", &token_shift);
   m.impl("rope_cache_write", &rope_cache_write);
   m.impl("multi_attention", &multi_attention);
+  m.impl("tile_attention", &tile_attention);
   m.impl("rglru_scan", &rglru_scan);
   m.impl("xielu", &xielu);
   m.impl("scale_rows", &scale_rows);

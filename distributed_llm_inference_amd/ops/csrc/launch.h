@@ -188,8 +188,8 @@ void dlia_par_norm(void* out, int out_f32, float* out32, float* x, const float* 
 void dlia_token_shift(void* out, int out_f32, const float* n32, const float* carry, const float* mu, const int* tok_pos,
                       const int* tok_seq, int T, int state_rows, int H, long ldo, hipStream_t stream);
 void dlia_rope_cache_write(float* q, long ldq, int q_vecs, int q_stride, int q_off, void* q_out, long ldqo, int q_cols, float* kv,
-                           long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols, void* kcache, void* vcache,
-                           int f32, int G, int dims, int interleaved, const float* cos_t, const float* sin_t, int table_pos,
+                           long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols, int v_t, void* kcache,
+                           void* vcache, int f32, int G, int dims, int interleaved, const float* cos_t, const float* sin_t, int table_pos,
                            const int* tok_pos, const int* tok_seq, const int* block_table, int T, int max_blocks, int num_blocks,
                            int table_rows, hipStream_t stream);
 void dlia_multi_attention(void* out, long ldo, const float* q, long ldq, int q_head, const void* kcache, int k_row,
@@ -197,6 +197,12 @@ void dlia_multi_attention(void* out, long ldo, const float* q, long ldq, int q_h
                           const int* block_table, int T, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
                           int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
                           const float* gate, long ldg, hipStream_t stream);
+// bf16 on the matrix cores; values key-contiguous in `vt` [blocks, G, dv, 32]. Returns 1 (nothing launched) for sizes it does not take.
+int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head, const void* kcache, int k_row, const void* vt,
+                        const int* q_start, const int* ctx, const int* slots, const int* block_table, int B, int max_q,
+                        int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv, int maps, float scale,
+                        int window, int keep_first, float softcap, float lam, float post, float eps, const float* gate, long ldg,
+                        hipStream_t stream);
 void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg, const float* ypre,
                      long ldy, const float* clam, float* state, const int* q_start, const int* ctx, const int* slots, int B,
                      int max_q, int W, int bw, int state_rows, hipStream_t stream);

@@ -104,8 +104,9 @@ __device__ __forceinline__ void rotate_row(float* row, int n_vec, int stride, in
 template <typename T>
 __global__ __launch_bounds__(kParThreads) void rope_cache_write_kernel(
     float* __restrict__ q, long ldq, int q_vecs, int q_stride, int q_off, T* __restrict__ q_out, long ldqo, int q_cols,
-    float* __restrict__ kv, long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols, T* __restrict__ kcache,
-    T* __restrict__ vcache, int G, int dims, int interleaved, const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+    float* __restrict__ kv, long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols, int v_t,
+    T* __restrict__ kcache, T* __restrict__ vcache, int G, int dims, int interleaved, const float* __restrict__ cos_t,
+    const float* __restrict__ sin_t,
     int table_pos, const int* __restrict__ tok_pos, const int* __restrict__ tok_seq, const int* __restrict__ block_table,
     int max_blocks, int num_blocks, int table_rows) {
   const int t = blockIdx.x;
@@ -130,11 +131,13 @@ __global__ __launch_bounds__(kParThreads) void rope_cache_write_kernel(
     kcache[(((long)blk * G + g) * kParBlock + off) * dk + c] = (T)krow[i];
   }
   if (vcache) {
+    // values: entries [v_src, v_src + v_cols) of the row; v_t: a block holds them key-contiguous, [head][entry][32 tokens]
     const int dv = v_cols / G;
-    const float* vrow = krow + k_cols;
+    const float* vrow = krow + v_src;
     for (int i = threadIdx.x; i < v_cols; i += kParThreads) {
       const int g = i / dv, c = i % dv;
-      vcache[(((long)blk * G + g) * kParBlock + off) * dv + c] = (T)vrow[i];
+      if (v_t) vcache[(((long)blk * G + g) * dv + c) * kParBlock + off] = (T)vrow[i];
+      else vcache[(((long)blk * G + g) * kParBlock + off) * dv + c] = (T)vrow[i];
     }
   }
 }
@@ -286,6 +289,161 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
     }
 }
 
+
+// ---- attention on the matrix cores (bf16) ---------------------------------------------------------------------------
+// One wave per (16 consecutive tokens of a sequence, head). Per cache block of 32 keys: S^T = K . Q^T as two 16-key MFMA tiles
+// per score map (K fragments straight from the cache rows, Q fragments from LDS), so that a lane holds 8 scores of ONE query:
+// scale, cap, mask and the running softmax are lane-local up to two shuffles over the four lanes that share a query. The
+// weights of those 8 keys ARE the lane's B fragment of O^T += V^T . P^T when the A fragment takes the same keys in the same
+// order, which it can because values sit key-contiguous in the cache: two 8-byte loads per 16 value entries. Both maps of a
+// head use the same value fragments. Blocks in front of the window are skipped except those that hold kept first tokens.
+template <int MAPS, int DVT>
+__global__ __launch_bounds__(64) void tile_attention_kernel(
+    bf16* __restrict__ out, long ldo, const bf16* __restrict__ q, long ldq, int q_head, const bf16* __restrict__ kcache, int k_row,
+    const bf16* __restrict__ vt, const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots,
+    const int* __restrict__ block_table, int tiles_per_seq, int max_blocks, int num_blocks, int table_rows, int H, int G, int d,
+    int dv, float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
+    const float* __restrict__ gate, long ldg) {
+  extern __shared__ __attribute__((aligned(16))) bf16 qs[];            // [16][MAPS * d + 8]
+  const int b = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq, h = blockIdx.y, g = h / (H / G);
+  const int t0 = q_start[b], n = q_start[b + 1] - t0, c0 = ctx[b], slot = slots[b];
+  const int r0 = ti * 16;
+  if (r0 >= n || slot < 0 || slot >= table_rows) return;               // (whole wave)
+  const int nrows = min(16, n - r0);
+  const int lane = threadIdx.x, r16 = lane & 15, kq = lane >> 4;
+  const int qp = MAPS * d + 8, per_row = MAPS * d / 8;
+  for (int i = lane; i < 16 * per_row; i += 64) {
+    const int r = i / per_row, c8 = i % per_row;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (r < nrows) v = ld16(q + (long)(t0 + r0 + r) * ldq + (long)h * q_head + c8 * 8);
+    st16(qs + r * qp + c8 * 8, v);
+  }
+  __syncthreads();
+  const int pos_first = c0 + r0, pos_last = pos_first + nrows - 1;
+  const int qpos = pos_first + r16;
+  const bool qvalid = r16 < nrows;
+  const int* table = block_table + (long)slot * max_blocks;
+  float m[MAPS], lsum[MAPS];
+  f32x4 o[MAPS][DVT];
+#pragma unroll
+  for (int a = 0; a < MAPS; ++a) {
+    m[a] = -INFINITY; lsum[a] = 0.f;
+#pragma unroll
+    for (int c = 0; c < DVT; ++c) o[a][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+  const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
+  const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  const int kb_lo = lo_first / kParBlock, kb_hi = min(pos_last / kParBlock, max_blocks - 1);
+  const int kept = (window > 0 && keep_first > 0) ? min(keep_first, lo_first) : 0;
+  const int kb_kept = kept > 0 ? min((kept - 1) / kParBlock, kb_lo - 1) : -1;      // blocks [0, kb_kept] hold kept tokens only
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  for (int kb = kb_kept >= 0 ? 0 : kb_lo; kb <= kb_hi; kb = (kb == kb_kept ? kb_lo : kb + 1)) {
+    const int blk = table[kb];
+    if (blk < 0 || blk >= num_blocks) continue;                        // (uniform)
+    f32x4 s[MAPS][2];
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) s[a][0] = s[a][1] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16* kbase = kcache + ((long)blk * G + g) * kParBlock * k_row;
+    for (int k0 = 0; k0 < d; k0 += 32) {
+      const int k = k0 + kq * 8;
+      const bool kin = k < d;
+#pragma unroll
+      for (int a = 0; a < MAPS; ++a) {
+        const u32x4 bq = kin ? ld16(qs + r16 * qp + a * d + k) : zero;
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl) {
+          const u32x4 ak = kin ? ld16(kbase + (long)(tl * 16 + r16) * k_row + a * d + k) : zero;
+          s[a][tl] = mfma16(ak, bq, s[a][tl]);
+        }
+      }
+    }
+    u32x4 pf[MAPS];
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) {
+      float sv[8];
+      float bm = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int j = kb * kParBlock + (i >> 2) * 16 + kq * 4 + (i & 3);
+        const bool vis = qvalid && j <= qpos && (window <= 0 || qpos - j < window || j < keep_first);
+        float x = s[a][i >> 2][i & 3] * scale;
+        if (softcap > 0.f) x = softcap * tanhf(x * inv_cap);
+        sv[i] = vis ? x : -INFINITY;
+        bm = fmaxf(bm, sv[i]);
+      }
+      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float m_new = fmaxf(m[a], bm);
+      float p[8], corr = 1.f, add = 0.f;
+      if (m_new == -INFINITY) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) p[i] = 0.f;
+      } else {
+        corr = (m[a] == -INFINITY) ? 0.f : expf(m[a] - m_new);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { p[i] = sv[i] == -INFINITY ? 0.f : expf(sv[i] - m_new); add += p[i]; }
+      }
+      lsum[a] = lsum[a] * corr + add;
+      m[a] = m_new;
+#pragma unroll
+      for (int c = 0; c < DVT; ++c) o[a][c] *= corr;
+      pf[a] = pack8(p);
+    }
+    const bf16* vbase = vt + ((long)blk * G + g) * dv * kParBlock;
+#pragma unroll
+    for (int c = 0; c < DVT; ++c) {
+      if (c * 16 >= dv) break;
+      const int row = c * 16 + r16;
+      u32x4 av = zero;
+      if (row < dv) {
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(vbase + (long)row * kParBlock + kq * 4);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(vbase + (long)row * kParBlock + 16 + kq * 4);
+        av = u32x4{lo.x, lo.y, hi.x, hi.y};
+      }
+#pragma unroll
+      for (int a = 0; a < MAPS; ++a) o[a][c] = mfma16(av, pf[a], o[a][c]);
+    }
+  }
+  float inv[MAPS];
+#pragma unroll
+  for (int a = 0; a < MAPS; ++a) {
+    float l = lsum[a];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    inv[a] = l > 0.f ? 1.f / l : 0.f;
+  }
+  float mul = inv[0];
+  if constexpr (MAPS == 2) {
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < DVT; ++c)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float v = o[0][c][r] * inv[0] - lam * o[1][c][r] * inv[1];
+        o[0][c][r] = v;
+        ss += v * v;
+      }
+    ss += __shfl_xor(ss, 16, 64);
+    ss += __shfl_xor(ss, 32, 64);
+    mul = post / sqrtf(ss / dv + eps);
+  }
+  if (!qvalid) return;
+  const long t = t0 + r0 + r16;
+  bf16* orow = out + t * ldo + (long)h * dv;
+  const float* grow = gate ? gate + t * ldg + (long)h * dv : nullptr;
+#pragma unroll
+  for (int c = 0; c < DVT; ++c)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int col = c * 16 + kq * 4 + r;
+      if (col < dv) {
+        float v = o[0][c][r] * mul;
+        if (grow) v *= 1.f / (1.f + expf(-grow[col]));
+        orow[col] = (bf16)v;
+      }
+    }
+}
+
 // ---- real-gated linear recurrence ----------------------------------------------------------------------------------
 __device__ __forceinline__ float gelu_tanh32(float x) {
   const float u = 0.7978845608028654f * (x + 0.044715f * x * x * x);
@@ -395,20 +553,20 @@ extern "C" void dlia_token_shift(void* out, int out_f32, const float* n32, const
 }
 
 extern "C" void dlia_rope_cache_write(float* q, long ldq, int q_vecs, int q_stride, int q_off, void* q_out, long ldqo, int q_cols,
-                                      float* kv, long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_cols,
-                                      void* kcache, void* vcache, int f32, int G, int dims, int interleaved, const float* cos_t,
+                                      float* kv, long ldkv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols,
+                                      int v_t, void* kcache, void* vcache, int f32, int G, int dims, int interleaved, const float* cos_t,
                                       const float* sin_t, int table_pos, const int* tok_pos, const int* tok_seq,
                                       const int* block_table, int T, int max_blocks, int num_blocks, int table_rows,
                                       hipStream_t stream) {
   if (T <= 0) return;
   if (f32)
     hipLaunchKernelGGL(rope_cache_write_kernel<float>, dim3(T), dim3(kParThreads), 0, stream, q, ldq, q_vecs, q_stride, q_off,
-                       (float*)q_out, ldqo, q_cols, kv, ldkv, k_cols, k_vecs, k_stride, k_off, v_cols, (float*)kcache,
+                       (float*)q_out, ldqo, q_cols, kv, ldkv, k_cols, k_vecs, k_stride, k_off, v_src, v_cols, v_t, (float*)kcache,
                        (float*)vcache, G, dims, interleaved, cos_t, sin_t, table_pos, tok_pos, tok_seq, block_table, max_blocks,
                        num_blocks, table_rows);
   else
     hipLaunchKernelGGL(rope_cache_write_kernel<bf16>, dim3(T), dim3(kParThreads), 0, stream, q, ldq, q_vecs, q_stride, q_off,
-                       (bf16*)q_out, ldqo, q_cols, kv, ldkv, k_cols, k_vecs, k_stride, k_off, v_cols, (bf16*)kcache,
+                       (bf16*)q_out, ldqo, q_cols, kv, ldkv, k_cols, k_vecs, k_stride, k_off, v_src, v_cols, v_t, (bf16*)kcache,
                        (bf16*)vcache, G, dims, interleaved, cos_t, sin_t, table_pos, tok_pos, tok_seq, block_table, max_blocks,
                        num_blocks, table_rows);
 }
@@ -480,4 +638,28 @@ extern "C" void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStr
   const long n = (long)M * N;
   if (n <= 0) return;
   hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, M, N, ld, s);
+}
+
+extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head, const void* kcache, int k_row,
+                                   const void* vt, const int* q_start, const int* ctx, const int* slots, const int* block_table,
+                                   int B, int max_q, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
+                                   int maps, float scale, int window, int keep_first, float softcap, float lam, float post,
+                                   float eps, const float* gate, long ldg, hipStream_t stream) {
+  if (B <= 0 || max_q <= 0) return 0;
+  if (d % 8 || k_row % 8 || q_head % 8 || ldq % 8 || maps * d > 1024 || dv > 512 || (maps != 1 && maps != 2)) return 1;
+  const int tiles = (max_q + 15) / 16;
+  const dim3 grid(B * tiles, H);
+  const size_t lds = (size_t)16 * (maps * d + 8) * sizeof(bf16);
+#define DLIA_TILE(MAPS, DVT)                                                                                                   \
+  hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT>), grid, dim3(64), lds, stream, (bf16*)out, ldo, (const bf16*)q, ldq, q_head, \
+                     (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, tiles, max_blocks, num_blocks, \
+                     table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg)
+  const int dvt = dv <= 64 ? 4 : dv <= 128 ? 8 : dv <= 256 ? 16 : 32;
+  if (maps == 2) {
+    if (dvt == 4) DLIA_TILE(2, 4); else if (dvt == 8) DLIA_TILE(2, 8); else if (dvt == 16) DLIA_TILE(2, 16); else DLIA_TILE(2, 32);
+  } else {
+    if (dvt == 4) DLIA_TILE(1, 4); else if (dvt == 8) DLIA_TILE(1, 8); else if (dvt == 16) DLIA_TILE(1, 16); else DLIA_TILE(1, 32);
+  }
+#undef DLIA_TILE
+  return 0;
 }

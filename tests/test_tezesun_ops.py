@@ -188,7 +188,7 @@ def test_rotation_cache_write_and_attention_hip(dtype, H, G, d, dv, maps, window
         tok_pos, tok_seq, *_ = _meta([(1, n, t0)], dev)
         z = f(z_all[t0:t0 + n])
         out = torch.zeros(n, H * dv, device=dev, dtype=dtype)
-        K.rope_cache_write(z, H * maps, d, 0, None, 0, z[:, qn:], kn, G * maps, d, 0, vn, kc, vc, dims, inter, f(cos), f(sin), tok_pos, tok_seq, table)
+        K.rope_cache_write(z, H * maps, d, 0, None, 0, z[:, qn:], kn, G * maps, d, 0, kn, vn, False, kc, vc, dims, inter, f(cos), f(sin), tok_pos, tok_seq, table)
         K.multi_attention(out, z, maps * d, kc, vc, 0, tok_pos, tok_seq, table, H, d, dv, maps, scale, window, keep, cap, lam, post, eps,
                           f(gate[t0:t0 + n]) if maps == 2 else None)
         got.append(out.float().cpu())
@@ -253,3 +253,56 @@ def test_block_products_activation_and_scale_hip():
     ref[:, :25] *= 1.7
     K.scale_rows(lg, 25, 1.7)
     close(lg, ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,dv,maps,window,keep,cap,dims,inter", [
+    (4, 2, 16, 24, 2, 40, 5, 10.0, 8, True), (2, 1, 8, 8, 1, 0, 0, 0.0, 8, False), (3, 3, 24, 70, 2, 3, 50, 0.0, 4, True),
+    (2, 2, 72, 130, 1, 33, 0, 3.0, 0, False), (6, 1, 40, 16, 2, 64, 1, 25.0, 10, True), (1, 1, 104, 300, 1, 0, 0, 0.0, 16, False),
+    (2, 1, 48, 96, 2, 31, 33, 20.0, 12, True)])
+def test_tile_attention_hip(H, G, d, dv, maps, window, keep, cap, dims, inter):
+    """The matrix-core attention kernel (bf16, values key-contiguous in the cache) on two sequences that share steps with
+    different portions (down to single tokens), blocks in no order, against whole-sequence attention."""
+    K, dev, dtype = _K(), "cuda", torch.bfloat16
+    T, eps, lam, post, scale = 150, 1e-5, 0.37, 0.6, 0.3
+    q, k = rnd(T, H * maps, d, seed=1), rnd(T, G * maps, d, seed=2)
+    v, gate = rnd(T, G, dv, seed=3).bfloat16().to(F64), rnd(T, H * dv, seed=4)
+    cos, sin = O.rope_angles({"dims": dims, "base": 50.0}, T) if dims else (None, None)
+    qr, kr = (O.rotate(q, cos, sin, inter), O.rotate(k, cos, sin, inter)) if dims else (q, k)
+    qr, kr = qr.bfloat16().to(F64), kr.bfloat16().to(F64)          # (what the kernel reads: rotated in fp32, then rounded)
+    ok = O.visible(T, window, keep)
+    heads = []
+    for hh in range(H):
+        g, per = hh // (H // G), []
+        for mp in range(maps):
+            s = (qr[:, maps * hh + mp] @ kr[:, maps * g + mp].T) * scale
+            if cap > 0:
+                s = cap * torch.tanh(s / cap)
+            per.append(torch.softmax(s.masked_fill(~ok, float("-inf")), -1) @ v[:, g])
+        heads.append(O.rms(per[0] - lam * per[1], eps) * post if maps == 2 else per[0])
+    ref = torch.cat(heads, -1) * (torch.sigmoid(gate) if maps == 2 else 1.0)
+    nblk = 12
+    kc = torch.zeros(nblk, G, 32, maps * d, device=dev, dtype=dtype)
+    vt = torch.zeros(nblk, G, dv, 32, device=dev, dtype=dtype)
+    table = torch.full((3, 6), -1, dtype=torch.int32, device=dev)
+    table[1, :5] = torch.tensor([7, 2, 5, 0, 3], dtype=torch.int32)
+    table[2, :5] = torch.tensor([11, 1, 9, 4, 6], dtype=torch.int32)
+    f = lambda t: t.float().to(dev).contiguous() if t is not None else None
+    z_all = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1)
+    qn, kn, vn = H * maps * d, G * maps * d, G * dv
+    got_a, got_b, a0, b0 = [], [], 0, 0
+    for na, nb in zip((50, 47, 1, 1, 1, 50), (1, 20, 30, 33, 2, 64)):
+        tok_pos, tok_seq, q_start, ctx, slots = _meta([(2, nb, b0), (1, na, a0)], dev)
+        z = f(torch.cat([z_all[b0:b0 + nb], z_all[a0:a0 + na]]))
+        gt = f(torch.cat([gate[b0:b0 + nb], gate[a0:a0 + na]]))
+        n = na + nb
+        out, q16 = torch.zeros(n, H * dv, device=dev, dtype=dtype), torch.zeros(n, qn, device=dev, dtype=dtype)
+        K.rope_cache_write(z, H * maps, d, 0, q16, qn, z[:, qn:], kn, G * maps, d, 0, kn, vn, True, kc, vt, dims, inter, f(cos), f(sin),
+                           tok_pos, tok_seq, table)
+        K.tile_attention(out, q16, maps * d, kc, vt, q_start, ctx, slots, table, max(na, nb), H, d, dv, maps, scale, window, keep, cap, lam,
+                         post, eps, gt if maps == 2 else None)
+        got_b.append(out[:nb].float().cpu())
+        got_a.append(out[nb:].float().cpu())
+        a0, b0 = a0 + na, b0 + nb
+    close(torch.cat(got_a), ref, 2e-2)
+    close(torch.cat(got_b), ref, 2e-2)
