@@ -144,8 +144,10 @@ class HybridGpuStage(GpuStage):
             # attention layers whose sizes are multiples of 8 run on the matrix cores in bf16 (values key-contiguous in the
             # cache); other sizes, and the fp32 mode, on the one-wave-per-(token, head) kernel. DLIA_PAR_TILE_ATTN=0: all on that (A/B)
             tile_ok = dtype == "bf16" and os.environ.get("DLIA_PAR_TILE_ATTN", "1") != "0"
-            self._tile = [tile_ok and ls.kind != "rglru" and self._score_dim(ls) % 8 == 0 and ls.maps * self._score_dim(ls) <= 1024
-                          for ls in self.specs]
+            def fits(ls):        # (sizes in whole 16-byte pieces, a query tile within a workgroup's LDS, accumulators within the registers)
+                d, dv = self._score_dim(ls), ls.kv_rank if ls.kind == "latent_attention" else ls.vdim
+                return d % 8 == 0 and ls.maps * d <= 1024 and dv <= (128 if ls.maps == 2 else 512)
+            self._tile = [tile_ok and ls.kind != "rglru" and fits(ls) for ls in self.specs]
             self._load_par(weights, f32, mat)
         elif self.gated:
             self._load_gated(weights, f32, mat)
@@ -738,7 +740,13 @@ class HybridGpuStage(GpuStage):
             for m_ in {rows, min(rows, 512), min(rows, 1024)}:
                 if m_ > self.decode_rows:
                     ws_floats = max([ws_floats] + [int(self.K.gemm_ws_floats(m_, n_, k_)) for n_, k_, _ in self._shapes])
+        part = 1                  # partial results of the key splits of single-token steps (any number of rows up to B)
+        for ls, tile in zip(self.specs, self._tile):
+            if tile:
+                dv = ls.kv_rank if ls.kind == "latent_attention" else ls.vdim
+                part = max([part] + [int(self.K.tile_attention_part_floats(b_, ls.heads, ls.kv_heads, dv, ls.maps)) for b_ in range(1, B + 1)])
         return SimpleNamespace(
+            part=z(part),
             h=torch.zeros(rows, H, device=dev), n32=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at),
             xs=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc), u=z(rows * uc), gates=z(rows * 2 * uc), mixed=z(rows * mc, at),
             ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2), act=z(rows * ac, at), cq=z(rows * cq, at), q32=z(rows * q32),
@@ -776,7 +784,7 @@ class HybridGpuStage(GpuStage):
                     K.rope_cache_write(z, Hh * M, d, 0, q16, qn, z[:, qn:], kn, G * M, d, 0, kn, vn, True, kc, vc, ls.rope_dims,
                                        ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
                     K.tile_attention(mixed, q16, M * d, kc, vc, q_start, ctx, slots, table, max_q, Hh, d, dv, M, ls.scale, ls.window or 0,
-                                     ls.keep_first, ls.softcap, p["lam"], post, eps, gate)
+                                     ls.keep_first, ls.softcap, p["lam"], post, eps, gate, wk.part)
                 else:
                     K.rope_cache_write(z, Hh * M, d, 0, None, 0, z[:, qn:], kn, G * M, d, 0, kn, vn, False, kc, vc, ls.rope_dims,
                                        ls.rope_interleaved, p["cos"], p["sin"], tok_pos, tok_seq, table)
@@ -797,7 +805,7 @@ class HybridGpuStage(GpuStage):
                     qa16 = view(wk.qa16, Hh * (R + dr))
                     K.gemm_blocks(qa16, q16, p["w_abs"], None, d + dr, R + dr)
                     K.tile_attention(olat, qa16, R + dr, kc, vc, q_start, ctx, slots, table, max_q, Hh, R + dr, R, 1, ls.scale, 0, 0, 0.0,
-                                     0.0, 1.0, eps, None)
+                                     0.0, 1.0, eps, None, wk.part)
                 else:
                     K.gemm_blocks(qa, q16, p["w_abs"], None, d + dr, R + dr)
                     K.multi_attention(olat, qa, R + dr, kc, kc, 0, tok_pos, tok_seq, table, Hh, R + dr, R, 1, ls.scale, 0, 0, 0.0, 0.0, 1.0,

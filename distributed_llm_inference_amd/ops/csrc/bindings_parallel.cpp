@@ -180,7 +180,7 @@ void multi_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& 
 void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& kcache, const Tensor& vt, const Tensor& q_start,
                     const Tensor& ctx, const Tensor& slots, const Tensor& block_table, int64_t max_q, int64_t H, int64_t d, int64_t dv,
                     int64_t maps, double scale, int64_t window, int64_t keep_first, double softcap, double lam, double post, double eps,
-                    OptTensor gate) {
+                    OptTensor gate, const std::optional<Tensor>& part) {
   DLIA_ON_DEVICE_OF(out);
   check_mat(out, "out"); check_mat(q, "q");
   check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots"); check_i32(block_table, "block_table");
@@ -201,12 +201,20 @@ void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& k
     DLIA_CHECK(gate->size(0) >= T && gate->size(1) == H * dv, "tile_attention: gate [T, H * dv]");
     gp = gate->data_ptr<float>(); ldg = gate->stride(0);
   }
+  float* pp = nullptr; long pn = 0;
+  if (part.has_value()) { check_f32(*part, "part"); pp = part->data_ptr<float>(); pn = part->numel(); }
+  DLIA_CHECK(max_q != 1 || T == B, "tile_attention: a single-token step has one row per sequence");
   const int rc = dlia_tile_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), (int)q_head, kcache.data_ptr(), (int)k_row,
                                      vt.data_ptr(), q_start.data_ptr<int>(), ctx.data_ptr<int>(), slots.data_ptr<int>(), block_table.data_ptr<int>(),
                                      (int)B, (int)max_q, (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0), (int)H, (int)G,
                                      (int)d, (int)dv, (int)maps, (float)scale, (int)window, (int)keep_first, (float)softcap, (float)lam,
-                                     (float)post, (float)eps, gp, ldg, cur_stream());
+                                     (float)post, (float)eps, gp, ldg, pp, pn, cur_stream());
+  DLIA_CHECK(rc != 2, "tile_attention: a single-token step needs the workspace for its key splits (tile_attention_part_floats)");
   DLIA_CHECK(rc == 0, "tile_attention: sizes must be multiples of 8 (d, key row, q head stride, q row), maps * d <= 1024, dv <= 512");
+}
+
+int64_t tile_attention_part_floats(int64_t B, int64_t H, int64_t G, int64_t dv, int64_t maps) {
+  return B * H * maps * dlia_tile_attention_splits((int)B, (int)H, (int)G) * (dv + 2);
 }
 
 // out [T, W] = S_t * gelu_tanh(ypre); u [T, W] conv output, gates [T, blocks * 2 bw] (per block: the decay gate's bw logits, then
@@ -260,7 +268,8 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("token_shift(Tensor(a!) out, Tensor n32, Tensor carry, Tensor mu, Tensor tok_pos, Tensor tok_seq) -> ()");
   m.def("rope_cache_write(Tensor(a!) q, int q_vecs, int q_stride, int q_off, Tensor(b!)? q_out, int q_cols, Tensor(c!) kv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols, bool v_t, Tensor(d!) kcache, Tensor(e!)? vcache, int dims, bool interleaved, Tensor? cos_t, Tensor? sin_t, Tensor tok_pos, Tensor tok_seq, Tensor block_table) -> ()");
   m.def("multi_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vcache, int v_off, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate) -> ()");
-  m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate) -> ()");
+  m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, Tensor(b!)? part) -> ()");
+  m.def("tile_attention_part_floats(int B, int H, int G, int dv, int maps) -> int");
   m.def("rglru_scan(Tensor(a!) out, Tensor u, Tensor gates, Tensor ypre, Tensor clam, Tensor(b!) state, Tensor q_start, Tensor ctx, Tensor slots, int bw, int max_q) -> ()");
   m.def("xielu(Tensor(a!) act, Tensor z, Tensor pq) -> ()");
   m.def("scale_rows(Tensor(a!) x, int cols, float s) -> ()");
@@ -277,4 +286,8 @@ TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
   m.impl("xielu", &xielu);
   m.impl("scale_rows", &scale_rows);
   m.impl("gemm_blocks", &gemm_blocks);
+}
+
+TORCH_LIBRARY_IMPL(dlia, CompositeExplicitAutograd, m) {
+  m.impl("tile_attention_part_floats", &tile_attention_part_floats);
 }

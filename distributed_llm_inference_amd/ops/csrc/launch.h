@@ -202,7 +202,9 @@ int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head
                         const int* q_start, const int* ctx, const int* slots, const int* block_table, int B, int max_q,
                         int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv, int maps, float scale,
                         int window, int keep_first, float softcap, float lam, float post, float eps, const float* gate, long ldg,
-                        hipStream_t stream);
+                        float* part, long part_floats, hipStream_t stream);
+// key splits of a single-token step of B rows (the workspace `part` holds B * H * maps * splits * (dv + 2) floats)
+int dlia_tile_attention_splits(int B, int H, int G);
 void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg, const float* ypre,
                      long ldy, const float* clam, float* state, const int* q_start, const int* ctx, const int* slots, int B,
                      int max_q, int W, int bw, int state_rows, hipStream_t stream);

@@ -297,30 +297,50 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
 // weights of those 8 keys ARE the lane's B fragment of O^T += V^T . P^T when the A fragment takes the same keys in the same
 // order, which it can because values sit key-contiguous in the cache: two 8-byte loads per 16 value entries. Both maps of a
 // head use the same value fragments. Blocks in front of the window are skipped except those that hold kept first tokens.
-template <int MAPS, int DVT>
-__global__ __launch_bounds__(64) void tile_attention_kernel(
+template <int MAPS, int DVT, bool HEADROWS>
+__global__ __launch_bounds__(256) void tile_attention_kernel(
     bf16* __restrict__ out, long ldo, const bf16* __restrict__ q, long ldq, int q_head, const bf16* __restrict__ kcache, int k_row,
     const bf16* __restrict__ vt, const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots,
     const int* __restrict__ block_table, int tiles_per_seq, int max_blocks, int num_blocks, int table_rows, int H, int G, int d,
     int dv, float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
-    const float* __restrict__ gate, long ldg) {
-  extern __shared__ __attribute__((aligned(16))) bf16 qs[];            // [16][MAPS * d + 8]
-  const int b = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq, h = blockIdx.y, g = h / (H / G);
+    const float* __restrict__ gate, long ldg, float* __restrict__ part) {
+  extern __shared__ __attribute__((aligned(16))) bf16 qs_all[];        // per wave [16][MAPS * d + 8]
+  // Rows of a wave's tile. Prompt portions: 16 consecutive tokens of one head; the waves of a workgroup take neighbouring heads
+  // (those of one key / value head first), so the key and value fragments they all read come from L1 after the first.
+  // HEADROWS (steps of single tokens): the rows are the heads that share a key / value head, for ONE token: its keys and
+  // values are read once for all of them. The token's key blocks are dealt out to gridDim.z workgroups, each of which leaves
+  // its (maximum, sum, weighted values) in `part`; tile_merge_kernel folds them and finishes the heads.
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r16 = lane & 15, kq = lane >> 4;
+  const int group = H / G;
+  const int b = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq;
   const int t0 = q_start[b], n = q_start[b + 1] - t0, c0 = ctx[b], slot = slots[b];
-  const int r0 = ti * 16;
-  if (r0 >= n || slot < 0 || slot >= table_rows) return;               // (whole wave)
-  const int nrows = min(16, n - r0);
-  const int lane = threadIdx.x, r16 = lane & 15, kq = lane >> 4;
+  int h, g, r0, nrows;
+  if constexpr (HEADROWS) {
+    const int gt = (group + 15) / 16;
+    g = blockIdx.y / gt;
+    h = g * group + (blockIdx.y % gt) * 16;                             // head of row 0
+    r0 = 0;
+    nrows = n > 0 ? min(16, group - (blockIdx.y % gt) * 16) : 0;
+  } else {
+    h = blockIdx.y * (blockDim.x >> 6) + wave;
+    g = h < H ? h / group : 0;
+    r0 = ti * 16;
+    nrows = h < H ? min(16, n - r0) : 0;
+  }
+  if (nrows <= 0 || slot < 0 || slot >= table_rows) return;             // (whole wave; nothing below synchronises across waves)
   const int qp = MAPS * d + 8, per_row = MAPS * d / 8;
+  bf16* qs = qs_all + (long)wave * 16 * qp;
   for (int i = lane; i < 16 * per_row; i += 64) {
     const int r = i / per_row, c8 = i % per_row;
     u32x4 v = {0u, 0u, 0u, 0u};
-    if (r < nrows) v = ld16(q + (long)(t0 + r0 + r) * ldq + (long)h * q_head + c8 * 8);
+    if (r < nrows) v = ld16(q + (long)(HEADROWS ? t0 : t0 + r0 + r) * ldq + (long)(HEADROWS ? h + r : h) * q_head + c8 * 8);
     st16(qs + r * qp + c8 * 8, v);
   }
-  __syncthreads();
-  const int pos_first = c0 + r0, pos_last = pos_first + nrows - 1;
-  const int qpos = pos_first + r16;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int pos_first = c0 + r0, pos_last = HEADROWS ? pos_first : pos_first + nrows - 1;
+  const int qpos = HEADROWS ? pos_first : pos_first + r16;
   const bool qvalid = r16 < nrows;
   const int* table = block_table + (long)slot * max_blocks;
   float m[MAPS], lsum[MAPS];
@@ -337,25 +357,37 @@ __global__ __launch_bounds__(64) void tile_attention_kernel(
   const int kept = (window > 0 && keep_first > 0) ? min(keep_first, lo_first) : 0;
   const int kb_kept = kept > 0 ? min((kept - 1) / kParBlock, kb_lo - 1) : -1;      // blocks [0, kb_kept] hold kept tokens only
   const u32x4 zero = {0u, 0u, 0u, 0u};
+  int turn = 0;
   for (int kb = kb_kept >= 0 ? 0 : kb_lo; kb <= kb_hi; kb = (kb == kb_kept ? kb_lo : kb + 1)) {
+    if constexpr (HEADROWS) {
+      if ((turn++) % (int)gridDim.z != (int)blockIdx.z) continue;
+    }
     const int blk = table[kb];
     if (blk < 0 || blk >= num_blocks) continue;                        // (uniform)
     f32x4 s[MAPS][2];
 #pragma unroll
     for (int a = 0; a < MAPS; ++a) s[a][0] = s[a][1] = f32x4{0.f, 0.f, 0.f, 0.f};
     const bf16* kbase = kcache + ((long)blk * G + g) * kParBlock * k_row;
-    for (int k0 = 0; k0 < d; k0 += 32) {
-      const int k = k0 + kq * 8;
-      const bool kin = k < d;
+    for (int k0 = 0; k0 < d; k0 += 128) {
+      u32x4 ak[MAPS][4][2];
 #pragma unroll
-      for (int a = 0; a < MAPS; ++a) {
-        const u32x4 bq = kin ? ld16(qs + r16 * qp + a * d + k) : zero;
+      for (int a = 0; a < MAPS; ++a)
 #pragma unroll
-        for (int tl = 0; tl < 2; ++tl) {
-          const u32x4 ak = kin ? ld16(kbase + (long)(tl * 16 + r16) * k_row + a * d + k) : zero;
-          s[a][tl] = mfma16(ak, bq, s[a][tl]);
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int tl = 0; tl < 2; ++tl) {
+            const int k = k0 + u * 32 + kq * 8;
+            ak[a][u][tl] = k < d ? ld16(kbase + (long)(tl * 16 + r16) * k_row + a * d + k) : zero;
+          }
+#pragma unroll
+      for (int a = 0; a < MAPS; ++a)
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int k = k0 + u * 32 + kq * 8;
+          const u32x4 bq = k < d ? ld16(qs + r16 * qp + a * d + k) : zero;
+          s[a][0] = mfma16(ak[a][u][0], bq, s[a][0]);
+          s[a][1] = mfma16(ak[a][u][1], bq, s[a][1]);
         }
-      }
     }
     u32x4 pf[MAPS];
 #pragma unroll
@@ -410,8 +442,27 @@ __global__ __launch_bounds__(64) void tile_attention_kernel(
     float l = lsum[a];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
-    inv[a] = l > 0.f ? 1.f / l : 0.f;
+    lsum[a] = l;
   }
+  if constexpr (HEADROWS) {
+    if (!qvalid) return;
+    const int nz = gridDim.z;
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) {
+      float* pr = part + ((((long)t0 * H + h + r16) * MAPS + a) * nz + blockIdx.z) * (dv + 2);
+      if (kq == 0) { pr[dv] = m[a]; pr[dv + 1] = lsum[a]; }
+#pragma unroll
+      for (int c = 0; c < DVT; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int col = c * 16 + kq * 4 + r;
+          if (col < dv) pr[col] = o[a][c][r];
+        }
+    }
+    return;
+  }
+#pragma unroll
+  for (int a = 0; a < MAPS; ++a) inv[a] = lsum[a] > 0.f ? 1.f / lsum[a] : 0.f;
   float mul = inv[0];
   if constexpr (MAPS == 2) {
     float ss = 0.f;
@@ -428,9 +479,10 @@ __global__ __launch_bounds__(64) void tile_attention_kernel(
     mul = post / sqrtf(ss / dv + eps);
   }
   if (!qvalid) return;
-  const long t = t0 + r0 + r16;
-  bf16* orow = out + t * ldo + (long)h * dv;
-  const float* grow = gate ? gate + t * ldg + (long)h * dv : nullptr;
+  const long t = HEADROWS ? t0 : t0 + r0 + r16;
+  const int hr = HEADROWS ? h + r16 : h;
+  bf16* orow = out + t * ldo + (long)hr * dv;
+  const float* grow = gate ? gate + t * ldg + (long)hr * dv : nullptr;
 #pragma unroll
   for (int c = 0; c < DVT; ++c)
 #pragma unroll
@@ -442,6 +494,58 @@ __global__ __launch_bounds__(64) void tile_attention_kernel(
         orow[col] = (bf16)v;
       }
     }
+}
+
+
+// Folds the partial results of tile_attention_kernel's key splits for the heads of single-token rows and finishes them:
+// normalisation, the two maps combined and RMS-normed, the gate. One wave per (token, head).
+template <int MAPS>
+__global__ __launch_bounds__(256) void tile_merge_kernel(bf16* __restrict__ out, long ldo, const float* __restrict__ part, int items,
+                                                         int H, int dv, int nz, float lam, float post, float eps,
+                                                         const float* __restrict__ gate, long ldg) {
+  const int item = blockIdx.x * 4 + (threadIdx.x >> 6), lane = lane_id();
+  if (item >= items) return;
+  const int t = item / H, h = item % H;
+  float o[MAPS][kMultiMaxDV / 64];
+#pragma unroll
+  for (int a = 0; a < MAPS; ++a) {
+    const float* pr = part + (((long)t * H + h) * MAPS + a) * nz * (dv + 2);
+    float M = -INFINITY;
+    for (int z = 0; z < nz; ++z) M = fmaxf(M, pr[(long)z * (dv + 2) + dv]);
+    float L = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) o[a][c] = 0.f;
+    for (int z = 0; z < nz; ++z) {
+      const float* pz = pr + (long)z * (dv + 2);
+      const float mz = pz[dv];
+      if (mz == -INFINITY) continue;                  // (uniform: a split that saw no key)
+      const float w = expf(mz - M);
+      L += pz[dv + 1] * w;
+#pragma unroll
+      for (int c = 0; c < kMultiMaxDV / 64; ++c) { const int col = c * 64 + lane; if (col < dv) o[a][c] += pz[col] * w; }
+    }
+    const float inv = L > 0.f ? 1.f / L : 0.f;
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) o[a][c] *= inv;
+  }
+  float mul = 1.f;
+  if constexpr (MAPS == 2) {
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < kMultiMaxDV / 64; ++c) { o[0][c] -= lam * o[1][c]; ss += o[0][c] * o[0][c]; }
+    ss = wave_sum(ss);
+    mul = post / sqrtf(ss / dv + eps);
+  }
+  bf16* orow = out + (long)t * ldo + (long)h * dv;
+#pragma unroll
+  for (int c = 0; c < kMultiMaxDV / 64; ++c) {
+    const int col = c * 64 + lane;
+    if (col < dv) {
+      float v = o[0][c] * mul;
+      if (gate) v *= 1.f / (1.f + expf(-gate[(long)t * ldg + (long)h * dv + col]));
+      orow[col] = (bf16)v;
+    }
+  }
 }
 
 // ---- real-gated linear recurrence ----------------------------------------------------------------------------------
@@ -640,25 +744,57 @@ extern "C" void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStr
   hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, M, N, ld, s);
 }
 
+extern "C" int dlia_tile_attention_splits(int B, int H, int G) {
+  // single-token steps: enough workgroups for the chip whatever the batch (a token's key blocks are dealt out to them)
+  const int per = B * G * ((H / G + 15) / 16);
+  int z = 1;
+  while (z < 16 && per * z < 1024) z <<= 1;
+  return z;
+}
+
 extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head, const void* kcache, int k_row,
                                    const void* vt, const int* q_start, const int* ctx, const int* slots, const int* block_table,
                                    int B, int max_q, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
                                    int maps, float scale, int window, int keep_first, float softcap, float lam, float post,
-                                   float eps, const float* gate, long ldg, hipStream_t stream) {
+                                   float eps, const float* gate, long ldg, float* part, long part_floats, hipStream_t stream) {
   if (B <= 0 || max_q <= 0) return 0;
   if (d % 8 || k_row % 8 || q_head % 8 || ldq % 8 || maps * d > 1024 || dv > 512 || (maps != 1 && maps != 2)) return 1;
-  const int tiles = (max_q + 15) / 16;
-  const dim3 grid(B * tiles, H);
-  const size_t lds = (size_t)16 * (maps * d + 8) * sizeof(bf16);
-#define DLIA_TILE(MAPS, DVT)                                                                                                   \
-  hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT>), grid, dim3(64), lds, stream, (bf16*)out, ldo, (const bf16*)q, ldq, q_head, \
-                     (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, tiles, max_blocks, num_blocks, \
-                     table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg)
+  const bool head_rows = max_q == 1;
+  const int tiles = (max_q + 15) / 16, group = H / G;
   const int dvt = dv <= 64 ? 4 : dv <= 128 ? 8 : dv <= 256 ? 16 : 32;
+  const size_t qtile = (size_t)16 * (maps * d + 8) * sizeof(bf16);
+  int nw = head_rows ? 1 : (group % 4 == 0 || G == 1) && H >= 4 ? 4 : (group % 2 == 0 && H >= 2 ? 2 : 1);
+  while (nw > 1 && nw * qtile > 65536) nw >>= 1;           // (a workgroup's LDS)
+  const int nz = head_rows ? dlia_tile_attention_splits(B, H, G) : 1;
+  const dim3 grid(B * tiles, head_rows ? G * ((group + 15) / 16) : (H + nw - 1) / nw, nz);
+  const size_t lds = nw * qtile;
+  if (lds > 65536) return 1;
+  if (head_rows && (!part || part_floats < (long)B * H * maps * nz * (dv + 2))) return 2;
+#define DLIA_TILE(MAPS, DVT)                                                                                                     \
+  do {                                                                                                                           \
+    if (head_rows)                                                                                                               \
+      hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, true>), grid, dim3(64), lds, stream, (bf16*)out, ldo, (const bf16*)q, ldq, \
+                         q_head, (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, tiles, max_blocks,   \
+                         num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, part);  \
+    else                                                                                                                         \
+      hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, false>), grid, dim3(64 * nw), lds, stream, (bf16*)out, ldo,              \
+                         (const bf16*)q, ldq, q_head, (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, \
+                         tiles, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps,  \
+                         gate, ldg, part);                                                                                       \
+  } while (0)
   if (maps == 2) {
     if (dvt == 4) DLIA_TILE(2, 4); else if (dvt == 8) DLIA_TILE(2, 8); else if (dvt == 16) DLIA_TILE(2, 16); else DLIA_TILE(2, 32);
   } else {
     if (dvt == 4) DLIA_TILE(1, 4); else if (dvt == 8) DLIA_TILE(1, 8); else if (dvt == 16) DLIA_TILE(1, 16); else DLIA_TILE(1, 32);
+  }
+  if (head_rows) {
+    const int items = B * H;
+    if (maps == 2)
+      hipLaunchKernelGGL(tile_merge_kernel<2>, dim3((items + 3) / 4), dim3(256), 0, stream, (bf16*)out, ldo, part, items, H, dv, nz, lam,
+                         post, eps, gate, ldg);
+    else
+      hipLaunchKernelGGL(tile_merge_kernel<1>, dim3((items + 3) / 4), dim3(256), 0, stream, (bf16*)out, ldo, part, items, H, dv, nz, lam,
+                         post, eps, gate, ldg);
   }
 #undef DLIA_TILE
   return 0;

@@ -291,7 +291,7 @@ def test_tile_attention_hip(H, G, d, dv, maps, window, keep, cap, dims, inter):
     z_all = torch.cat([q.reshape(T, -1), k.reshape(T, -1), v.reshape(T, -1)], 1)
     qn, kn, vn = H * maps * d, G * maps * d, G * dv
     got_a, got_b, a0, b0 = [], [], 0, 0
-    for na, nb in zip((50, 47, 1, 1, 1, 50), (1, 20, 30, 33, 2, 64)):
+    for na, nb in zip((50, 47, 1, 1, 1, 50), (1, 20, 30, 1, 34, 64)):      # (the fourth step brings single tokens only)
         tok_pos, tok_seq, q_start, ctx, slots = _meta([(2, nb, b0), (1, na, a0)], dev)
         z = f(torch.cat([z_all[b0:b0 + nb], z_all[a0:a0 + na]]))
         gt = f(torch.cat([gate[b0:b0 + nb], gate[a0:a0 + na]]))
@@ -299,8 +299,9 @@ def test_tile_attention_hip(H, G, d, dv, maps, window, keep, cap, dims, inter):
         out, q16 = torch.zeros(n, H * dv, device=dev, dtype=dtype), torch.zeros(n, qn, device=dev, dtype=dtype)
         K.rope_cache_write(z, H * maps, d, 0, q16, qn, z[:, qn:], kn, G * maps, d, 0, kn, vn, True, kc, vt, dims, inter, f(cos), f(sin),
                            tok_pos, tok_seq, table)
+        part = torch.zeros(int(K.tile_attention_part_floats(2, H, G, dv, maps)), device=dev)
         K.tile_attention(out, q16, maps * d, kc, vt, q_start, ctx, slots, table, max(na, nb), H, d, dv, maps, scale, window, keep, cap, lam,
-                         post, eps, gt if maps == 2 else None)
+                         post, eps, gt if maps == 2 else None, part)
         got_b.append(out[:nb].float().cpu())
         got_a.append(out[nb:].float().cpu())
         a0, b0 = a0 + na, b0 + nb
