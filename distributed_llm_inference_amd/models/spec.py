@@ -867,12 +867,12 @@ def tezesun_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
                     rec_width=width, blocks=blocks or heads, conv=conv, ff=ff, ff_kind="xielu")
     dm = max(2, head_dim // 2)
     att = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=dm, vdim=head_dim, window=window, keep_first=keep_first,
-                    scale=dm ** -0.5, softcap=30.0, maps=2, diff=0.5, out_gate=True, rope_dims=dm, rope_base=500000.0, rope_interleaved=True,
-                    rope_scaling=RopeScaling(factor=8.0, rope_type="yarn", beta_fast=32.0, beta_slow=1.0, original_max_position_embeddings=1024),
+                    scale=dm ** -0.5, softcap=30.0, maps=2, diff=0.5, out_gate=True, rope_dims=dm, rope_base=1000000.0, rope_interleaved=True,
+                    rope_scaling=RopeScaling(factor=4.0, rope_type="yarn", beta_fast=32.0, beta_slow=1.0, original_max_position_embeddings=4096),
                     ff=ff, ff_kind="xielu")
     lat = LayerSpec("latent_attention", heads=heads, kv_heads=1, dim=head_dim, vdim=head_dim, scale=(head_dim + rot_dim) ** -0.5,
                     q_rank=q_rank or max(8, width // 2), kv_rank=kv_rank or max(8, width // 8), rot_dim=rot_dim, rope_dims=rot_dim,
-                    rope_base=250000.0, ff=ff, ff_kind="xielu")
+                    rope_base=10000.0, ff=ff, ff_kind="xielu")
     kinds = {"r": rec, "a": att, "l": lat}
     layers = tuple(kinds[pattern[i % len(pattern)]] for i in range(num_layers))
     return ModelSpec(name=name, family="tezesun", num_layers=num_layers, hidden_size=width, num_heads=heads, num_kv_heads=kv_heads,
@@ -911,7 +911,7 @@ def _register_test_models():
                                                           loop=(1, 3, 2), max_position=512, rank=16, bias_rows=16, bias_max=200)
     BUILTIN_SPECS["tiny-tezesun-test"] = tezesun_spec("tiny-tezesun-test", 64, 4, 2, 16, 96, 4, window=12, vocab_size=320, conv=3, blocks=4,
                                                       q_rank=24, kv_rank=20, rot_dim=8, keep_first=3)
-    BUILTIN_SPECS["tiny-tezesun-gpu-test"] = tezesun_spec("tiny-tezesun-gpu-test", 128, 4, 2, 32, 256, 4, window=40, vocab_size=320, blocks=2,
+    BUILTIN_SPECS["tiny-tezesun-gpu-test"] = tezesun_spec("tiny-tezesun-gpu-test", 128, 4, 2, 32, 256, 4, window=36, vocab_size=320, blocks=2,
                                                           q_rank=48, kv_rank=40, rot_dim=16, keep_first=5)
     BUILTIN_SPECS["tiny-gpt2-gpu-test"] = tiny_spec(
         "gpt2", name="tiny-gpt2-gpu-test", hidden_size=256, num_heads=4, num_kv_heads=4, head_dim=64,

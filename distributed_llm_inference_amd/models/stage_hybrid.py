@@ -745,8 +745,9 @@ class HybridGpuStage(GpuStage):
             if tile:
                 dv = ls.kv_rank if ls.kind == "latent_attention" else ls.vdim
                 part = max([part] + [int(self.K.tile_attention_part_floats(b_, ls.heads, ls.kv_heads, dv, ls.maps)) for b_ in range(1, B + 1)])
+        scan = max([1] + [int(self.K.rglru_scan_ws_floats(rows, B, ls.rec_width)) for ls in self.specs if ls.kind == "rglru"])
         return SimpleNamespace(
-            part=z(part),
+            part=z(part), scan_ws=z(scan),
             h=torch.zeros(rows, H, device=dev), n32=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at),
             xs=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc), u=z(rows * uc), gates=z(rows * 2 * uc), mixed=z(rows * mc, at),
             ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2), act=z(rows * ac, at), cq=z(rows * cq, at), q32=z(rows * q32),
@@ -771,7 +772,7 @@ class HybridGpuStage(GpuStage):
                 u, gates, mixed = view(wk.u, W), view(wk.gates, 2 * W), view(wk.mixed, W)
                 K.short_conv_act(u, z[:, W:2 * W], self.rec[li][1], p["conv_w"], p["conv_b"], q_start, ctx, slots, max_q, False)
                 K.gemm_blocks(gates, u, p["w_g"], p["b_g"], bw, 2 * bw)
-                K.rglru_scan(mixed, u, gates, z[:, :W], p["clam"], self.rec[li][2], q_start, ctx, slots, bw, max_q)
+                K.rglru_scan(mixed, u, gates, z[:, :W], p["clam"], self.rec[li][2], q_start, ctx, slots, bw, max_q, wk.scan_ws)
             elif ls.kind == "attention":
                 Hh, G, d, dv, M = ls.heads, ls.kv_heads, ls.dim, ls.vdim, ls.maps
                 qn, kn, vn = Hh * M * d, G * M * d, G * dv

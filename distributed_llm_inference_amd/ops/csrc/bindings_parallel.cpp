@@ -213,6 +213,8 @@ void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& k
   DLIA_CHECK(rc == 0, "tile_attention: sizes must be multiples of 8 (d, key row, q head stride, q row), maps * d <= 1024, dv <= 512");
 }
 
+int64_t rglru_scan_ws_floats(int64_t rows, int64_t B, int64_t W) { return dlia_rglru_scan_ws_floats((int)rows, (int)B, (int)W); }
+
 int64_t tile_attention_part_floats(int64_t B, int64_t H, int64_t G, int64_t dv, int64_t maps) {
   return B * H * maps * dlia_tile_attention_splits((int)B, (int)H, (int)G) * (dv + 2);
 }
@@ -220,7 +222,7 @@ int64_t tile_attention_part_floats(int64_t B, int64_t H, int64_t G, int64_t dv, 
 // out [T, W] = S_t * gelu_tanh(ypre); u [T, W] conv output, gates [T, blocks * 2 bw] (per block: the decay gate's bw logits, then
 // the input gate's), clam [W] = c softplus(lam), state [slots, W].
 void rglru_scan(Tensor out, const Tensor& u, const Tensor& gates, const Tensor& ypre, const Tensor& clam, Tensor state,
-                const Tensor& q_start, const Tensor& ctx, const Tensor& slots, int64_t bw, int64_t max_q) {
+                const Tensor& q_start, const Tensor& ctx, const Tensor& slots, int64_t bw, int64_t max_q, const std::optional<Tensor>& ws) {
   DLIA_ON_DEVICE_OF(out);
   check_act(out, "out"); check_mat(out, "out"); check_fmat(u, "u"); check_fmat(gates, "gates"); check_fmat(ypre, "ypre");
   check_f32(clam, "clam"); check_f32(state, "state"); check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots");
@@ -228,9 +230,11 @@ void rglru_scan(Tensor out, const Tensor& u, const Tensor& gates, const Tensor& 
   DLIA_CHECK(bw >= 1 && W % bw == 0 && u.size(0) >= T && u.size(1) == W && gates.size(0) >= T && gates.size(1) == 2 * W &&
              ypre.size(0) >= T && ypre.size(1) == W && clam.numel() == W, "rglru_scan: u, ypre [T, W], gates [T, 2 W], clam [W]");
   DLIA_CHECK(state.dim() == 2 && state.size(1) == W && q_start.numel() >= B + 1 && slots.numel() >= B && max_q <= T, "rglru_scan: state [slots, W], q_start [B + 1]");
+  if (ws.has_value()) check_f32(*ws, "ws");
   dlia_rglru_scan(out.data_ptr(), is_f32(out), out.stride(0), u.data_ptr<float>(), u.stride(0), gates.data_ptr<float>(), gates.stride(0),
                   ypre.data_ptr<float>(), ypre.stride(0), clam.data_ptr<float>(), state.data_ptr<float>(), q_start.data_ptr<int>(),
-                  ctx.data_ptr<int>(), slots.data_ptr<int>(), (int)B, (int)max_q, (int)W, (int)bw, (int)state.size(0), cur_stream());
+                  ctx.data_ptr<int>(), slots.data_ptr<int>(), (int)B, (int)max_q, (int)W, (int)bw, (int)state.size(0),
+                  ws.has_value() ? ws->data_ptr<float>() : nullptr, ws.has_value() ? (long)ws->numel() : 0, (int)T, cur_stream());
 }
 
 void xielu(Tensor act, const Tensor& z, const Tensor& pq) {
@@ -270,7 +274,8 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("multi_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vcache, int v_off, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate) -> ()");
   m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, Tensor(b!)? part) -> ()");
   m.def("tile_attention_part_floats(int B, int H, int G, int dv, int maps) -> int");
-  m.def("rglru_scan(Tensor(a!) out, Tensor u, Tensor gates, Tensor ypre, Tensor clam, Tensor(b!) state, Tensor q_start, Tensor ctx, Tensor slots, int bw, int max_q) -> ()");
+  m.def("rglru_scan(Tensor(a!) out, Tensor u, Tensor gates, Tensor ypre, Tensor clam, Tensor(b!) state, Tensor q_start, Tensor ctx, Tensor slots, int bw, int max_q, Tensor(c!)? ws) -> ()");
+  m.def("rglru_scan_ws_floats(int rows, int B, int W) -> int");
   m.def("xielu(Tensor(a!) act, Tensor z, Tensor pq) -> ()");
   m.def("scale_rows(Tensor(a!) x, int cols, float s) -> ()");
   m.def("gemm_blocks(Tensor(a!) out, Tensor x, Tensor w, Tensor? bias, int x_step, int out_step) -> ()");
@@ -290,4 +295,5 @@ TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
 
 TORCH_LIBRARY_IMPL(dlia, CompositeExplicitAutograd, m) {
   m.impl("tile_attention_part_floats", &tile_attention_part_floats);
+  m.impl("rglru_scan_ws_floats", &rglru_scan_ws_floats);
 }

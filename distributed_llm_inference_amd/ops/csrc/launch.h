@@ -207,7 +207,8 @@ int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head
 int dlia_tile_attention_splits(int B, int H, int G);
 void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg, const float* ypre,
                      long ldy, const float* clam, float* state, const int* q_start, const int* ctx, const int* slots, int B,
-                     int max_q, int W, int bw, int state_rows, hipStream_t stream);
+                     int max_q, int W, int bw, int state_rows, float* ws, long ws_floats, int rows, hipStream_t stream);
+long dlia_rglru_scan_ws_floats(int rows, int B, int W);
 void dlia_xielu(void* act, int out_f32, const float* z, int M, int F, long ldz, long lda, const float* pq, hipStream_t stream);
 void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStream_t stream);
 // ---- misc.hip -------------------------------------------------------------------------

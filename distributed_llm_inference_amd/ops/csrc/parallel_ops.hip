@@ -16,8 +16,9 @@
 //                   walked at once over the shared values and combined as rms(a1 - lam a2) (1 - diff) sigmoid(gate).
 //                   Keys are rows of any length (a map is a slice of the row), values may be a slice of the key rows.
 //   rglru_scan      S <- a S + sqrt(1 - a^2) i u per channel with a = exp(-c r), r and i sigmoids of the block gates;
-//                   read-out S * gelu_tanh(y). Long portions are cut into segments that are scanned side by side and
-//                   joined through the segments' (decay product, offset) pairs.
+//                   read-out S * gelu_tanh(y). Long portions are cut into stretches that are scanned side by side and
+//                   joined through the stretches' (decay product, end value) pairs: inside a workgroup through LDS, or,
+//                   given a workspace, over workgroups through memory in two launches.
 //   xielu, scale_rows   the feed-forward's activation; logits times a constant
 // Everything is fp32 except what feeds a GEMM or sits in the cache (the compute type, bf16 or fp32).
 #include "common.h"
@@ -610,6 +611,54 @@ __global__ __launch_bounds__(64 * SEGS) void rglru_scan_kernel(
   if (on && r1 == n && r1 > r0) state[(long)slot * W + c] = S;
 }
 
+// Long portions over the whole chip: the step's tokens are cut into stretches of 64 per sequence, one single-wave workgroup per
+// (sequence, 64 channels, stretch). First launch: every stretch scanned from zero, its (decay product, end value) left in `ws`
+// (row: the stretch's place among all stretches of the step). Second launch: a stretch folds those of the stretches before it
+// onto the slot's state, scans again from there and writes; the stretch with the step's last token leaves the new state.
+constexpr int kScanStretch = 64;
+
+template <typename OT, bool APPLY>
+__global__ __launch_bounds__(64) void rglru_stretch_kernel(
+    OT* __restrict__ out, long ldo, const float* __restrict__ u, long ldu, const float* __restrict__ gates, long ldg,
+    const float* __restrict__ ypre, long ldy, const float* __restrict__ clam, float* __restrict__ state, float* __restrict__ ws,
+    const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots, int W, int bw, int state_rows) {
+  const int b = blockIdx.x, sg = blockIdx.z;
+  const int t0 = q_start[b], n = q_start[b + 1] - t0, c0 = ctx[b], slot = slots[b];
+  const int r0 = sg * kScanStretch;
+  if (r0 >= n || slot < 0 || slot >= state_rows) return;
+  const int r1 = min(n, r0 + kScanStretch);
+  const int c = blockIdx.y * 64 + threadIdx.x;
+  const bool on = c < W;
+  const int cc = on ? c : 0;
+  const int gcol = (cc / bw) * 2 * bw + cc % bw;
+  const float cl = clam[cc];
+  // this sequence's rows of ws (rows of different sequences never meet): the slot's state as the step found it, then a row per
+  // stretch. The second launch reads the old state from there: by then the slot may already hold the new one.
+  const long row0 = t0 / kScanStretch + 2 * b;
+  if constexpr (!APPLY) {
+    if (sg == 0 && on) ws[(row0 * W + c) * 2 + 1] = c0 > 0 ? state[(long)slot * W + c] : 0.f;
+    float A = 1.f, Bv = 0.f;
+    for (int r = r0; r < r1; ++r) {
+      const long t = t0 + r;
+      float a, bb;
+      rglru_terms(u[t * ldu + cc], gates[t * ldg + gcol], gates[t * ldg + gcol + bw], cl, a, bb);
+      A *= a; Bv = a * Bv + bb;
+    }
+    if (on) { ws[((row0 + 1 + sg) * W + c) * 2] = A; ws[((row0 + 1 + sg) * W + c) * 2 + 1] = Bv; }
+  } else {
+    float S = ws[(row0 * W + cc) * 2 + 1];
+    for (int k = 0; k < sg; ++k) S = ws[((row0 + 1 + k) * W + cc) * 2] * S + ws[((row0 + 1 + k) * W + cc) * 2 + 1];
+    for (int r = r0; r < r1; ++r) {
+      const long t = t0 + r;
+      float a, bb;
+      rglru_terms(u[t * ldu + cc], gates[t * ldg + gcol], gates[t * ldg + gcol + bw], cl, a, bb);
+      S = a * S + bb;
+      if (on) out[t * ldo + c] = (OT)(S * gelu_tanh32(ypre[t * ldy + c]));
+    }
+    if (on && r1 == n) state[(long)slot * W + c] = S;
+  }
+}
+
 // ---- activation, scaling ---------------------------------------------------------------------------------------------
 template <typename OT>
 __global__ __launch_bounds__(256) void xielu_kernel(OT* __restrict__ act, const float* __restrict__ z, int M, int F, long ldz,
@@ -711,10 +760,23 @@ extern "C" void dlia_multi_attention(void* out, long ldo, const float* q, long l
                              softcap, lam, post, eps, gate, ldg, vec);
 }
 
+extern "C" long dlia_rglru_scan_ws_floats(int rows, int B, int W) { return ((long)rows / kScanStretch + 2 * B + 2) * W * 2; }
+
 extern "C" void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg,
                                 const float* ypre, long ldy, const float* clam, float* state, const int* q_start, const int* ctx,
-                                const int* slots, int B, int max_q, int W, int bw, int state_rows, hipStream_t stream) {
+                                const int* slots, int B, int max_q, int W, int bw, int state_rows, float* ws, long ws_floats, int rows,
+                                hipStream_t stream) {
   if (B <= 0 || max_q <= 0) return;
+  if (max_q >= 128 && ws && ws_floats >= dlia_rglru_scan_ws_floats(rows, B, W)) {
+    const dim3 grid(B, (W + 63) / 64, (max_q + kScanStretch - 1) / kScanStretch);
+#define DLIA_STRETCH(OT, APPLY)                                                                                                \
+  hipLaunchKernelGGL((rglru_stretch_kernel<OT, APPLY>), grid, dim3(64), 0, stream, (OT*)out, ldo, u, ldu, gates, ldg, ypre, ldy, clam, \
+                     state, ws, q_start, ctx, slots, W, bw, state_rows)
+    if (out_f32) { DLIA_STRETCH(float, false); DLIA_STRETCH(float, true); }
+    else { DLIA_STRETCH(bf16, false); DLIA_STRETCH(bf16, true); }
+#undef DLIA_STRETCH
+    return;
+  }
   const dim3 grid(B, (W + 63) / 64);
 #define DLIA_RGLRU(OT, SEGS)                                                                                              \
   hipLaunchKernelGGL((rglru_scan_kernel<OT, SEGS>), grid, dim3(64 * SEGS), 0, stream, (OT*)out, ldo, u, ldu, gates, ldg, ypre, \

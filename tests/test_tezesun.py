@@ -269,11 +269,11 @@ def _random_stack(seed: int):
             rot = rng.choice([0, 2, dim // 2 // 2 * 2, dim // 2 * 2])
             layers.append(A(heads, kv, dim, rng.choice([8, 16, 24, 64, 96]), window=win, keep_first=rng.choice([0, 1, 4, 40]),
                             scale=rng.choice([dim ** -0.5, 0.2]), softcap=rng.choice([0.0, 5.0, 30.0]), diff=rng.choice([0.1, 0.5, 0.8]),
-                            rot_dims=rot, base=rng.choice([100.0, 10000.0, 500000.0]), scaling=rng.choice([None, YARN]) if rot else None, ff=ff))
+                            rot_dims=rot, base=rng.choice([100.0, 10000.0, 1000000.0]), scaling=rng.choice([None, YARN]) if rot else None, ff=ff))
         else:
             dr = rng.choice([2, 4, 8, 16, 24])
             layers.append(L(rng.choice([1, 2, 3, 4, 8]), rng.choice([4, 8, 16, 24, 32]), dr, rng.choice([8, 16, 20, 48]), rng.choice([8, 24, 64, 128]),
-                            rng.choice([8, 12, 32, 72]), base=rng.choice([100.0, 250000.0]), ff=ff))
+                            rng.choice([8, 12, 32, 72]), base=rng.choice([100.0, 50000.0]), ff=ff))
     cfg = make_config(layers, vocab=rng.choice([33, 64, 100, 257]), width=width, eps=rng.choice([1e-5, 1e-6]), logit_scale=rng.choice([1.0, 2.0, 0.7]))
     cuts, left = [], 110
     while left > 0:

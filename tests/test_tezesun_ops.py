@@ -39,7 +39,7 @@ def test_partial_rotation_and_scaled_frequencies(interleaved, dims, D):
     from distributed_llm_inference_amd.models.rope import rope_table
     from distributed_llm_inference_amd.models.spec import RopeScaling
     from distributed_llm_inference_amd.ops import reference as R
-    for sc in (None, {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}, {"factor": 8.0, "original": 1000, "fast": 32.0, "slow": 1.0}):
+    for sc in (None, {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}, {"factor": 6.0, "original": 1000, "fast": 24.0, "slow": 1.5}):
         rot = {"dims": dims, "base": 100.0, **({"scaling": sc} if sc else {})}
         rs = RopeScaling(factor=sc["factor"], rope_type="yarn", beta_fast=sc["fast"], beta_slow=sc["slow"],
                          original_max_position_embeddings=sc["original"]) if sc else None
@@ -197,8 +197,9 @@ def test_rotation_cache_write_and_attention_hip(dtype, H, G, d, dv, maps, window
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("over_workgroups", [False, True])
 @pytest.mark.parametrize("W,nb,taps", [(24, 3, 3), (16, 1, 1), (100, 100, 4), (320, 4, 2)])
-def test_recurrent_unit_hip(W, nb, taps):
+def test_recurrent_unit_hip(W, nb, taps, over_workgroups):
     """short_conv_act + gemm_blocks + rglru_scan: two sequences in one step (a long portion that is scanned in segments
     beside a single token), several steps, slots that held other values, against the whole sequences."""
     K, dev, H = _K(), "cuda", 12
@@ -221,7 +222,8 @@ def test_recurrent_unit_hip(W, nb, taps):
         u, gates, out = torch.zeros(n, W, device=dev), torch.zeros(n, 2 * W, device=dev), torch.zeros(n, W, device=dev)
         K.short_conv_act(u, z[:, W:], carry, f(w["conv"]), f(w["conv.b"]), q_start, ctx, slots, max(na, nb_), False)
         K.gemm_blocks(gates, u, wg, bg, bw, 2 * bw)
-        K.rglru_scan(out, u, gates, z[:, :W], clam, state, q_start, ctx, slots, bw, max(na, nb_))
+        ws = torch.zeros(int(K.rglru_scan_ws_floats(n, 2, W)), device=dev) if over_workgroups else None
+        K.rglru_scan(out, u, gates, z[:, :W], clam, state, q_start, ctx, slots, bw, max(na, nb_), ws)
         got_b.append(out[:nb_].cpu())
         got_a.append(out[nb_:].cpu())
         a0, b0 = a0 + na, b0 + nb_
@@ -259,7 +261,7 @@ def test_block_products_activation_and_scale_hip():
 @pytest.mark.parametrize("H,G,d,dv,maps,window,keep,cap,dims,inter", [
     (4, 2, 16, 24, 2, 40, 5, 10.0, 8, True), (2, 1, 8, 8, 1, 0, 0, 0.0, 8, False), (3, 3, 24, 70, 2, 3, 50, 0.0, 4, True),
     (2, 2, 72, 130, 1, 33, 0, 3.0, 0, False), (6, 1, 40, 16, 2, 64, 1, 25.0, 10, True), (1, 1, 104, 300, 1, 0, 0, 0.0, 16, False),
-    (2, 1, 48, 96, 2, 31, 33, 20.0, 12, True)])
+    (2, 1, 56, 80, 2, 31, 33, 12.0, 14, True)])
 def test_tile_attention_hip(H, G, d, dv, maps, window, keep, cap, dims, inter):
     """The matrix-core attention kernel (bf16, values key-contiguous in the cache) on two sequences that share steps with
     different portions (down to single tokens), blocks in no order, against whole-sequence attention."""

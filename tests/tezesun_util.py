@@ -116,6 +116,6 @@ STACKS = {
     "only_rglru": make_config([R(64, 4, 4), R(128, 8, 2, ff=32), R(32, 2, 3, ff=0)], vocab=64, width=64),
     "only_latent": make_config([L(3, 12, 4, 20, 24, 18, scale=0.4), L(1, 32, 16, 8, 40, 48, ff=0), L(4, 8, 2, 8, 8, 8)], vocab=51, width=40, logit_scale=0.5),
     # widths and inner sizes that the packed-weight GEMMs take in bf16 (multiples of 128)
-    "packed": make_config([L(4, 32, 16, 32, 128, 48), R(128, 2, 4, ff=128), A(4, 2, 32, 64, window=40, keep_first=4, softcap=20.0, rot_dims=16,
-                                                                              scaling=YARN, ff=256), R(256, 4, 3, ff=128)], vocab=90, width=128, logit_scale=2.0),
+    "packed": make_config([L(4, 32, 16, 32, 128, 48), R(128, 2, 4, ff=128), A(4, 2, 32, 64, window=44, keep_first=4, softcap=25.0, rot_dims=16,
+                                                                              scaling=YARN, ff=256), R(256, 4, 3, ff=128)], vocab=90, width=128, logit_scale=2.5),
 }
