@@ -298,7 +298,7 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
 // weights of those 8 keys ARE the lane's B fragment of O^T += V^T . P^T when the A fragment takes the same keys in the same
 // order, which it can because values sit key-contiguous in the cache: two 8-byte loads per 16 value entries. Both maps of a
 // head use the same value fragments. Blocks in front of the window are skipped except those that hold kept first tokens.
-template <int MAPS, int DVT, bool HEADROWS>
+template <int MAPS, int DVT, bool HEADROWS, int KS>
 __global__ __launch_bounds__(256) void tile_attention_kernel(
     bf16* __restrict__ out, long ldo, const bf16* __restrict__ q, long ldq, int q_head, const bf16* __restrict__ kcache, int k_row,
     const bf16* __restrict__ vt, const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots,
@@ -369,12 +369,12 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
 #pragma unroll
     for (int a = 0; a < MAPS; ++a) s[a][0] = s[a][1] = f32x4{0.f, 0.f, 0.f, 0.f};
     const bf16* kbase = kcache + ((long)blk * G + g) * kParBlock * k_row;
-    for (int k0 = 0; k0 < d; k0 += 128) {
-      u32x4 ak[MAPS][4][2];
+    for (int k0 = 0; k0 < d; k0 += 32 * KS) {
+      u32x4 ak[MAPS][KS][2];          // KS k-steps of key fragments in flight at once
 #pragma unroll
       for (int a = 0; a < MAPS; ++a)
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int u = 0; u < KS; ++u)
 #pragma unroll
           for (int tl = 0; tl < 2; ++tl) {
             const int k = k0 + u * 32 + kq * 8;
@@ -383,7 +383,7 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
 #pragma unroll
       for (int a = 0; a < MAPS; ++a)
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < KS; ++u) {
           const int k = k0 + u * 32 + kq * 8;
           const u32x4 bq = k < d ? ld16(qs + r16 * qp + a * d + k) : zero;
           s[a][0] = mfma16(ak[a][u][0], bq, s[a][0]);
@@ -832,17 +832,23 @@ extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq,
   const size_t lds = nw * qtile;
   if (lds > 65536) return 1;
   if (head_rows && (!part || part_floats < (long)B * H * maps * nz * (dv + 2))) return 2;
-#define DLIA_TILE(MAPS, DVT)                                                                                                     \
+#define DLIA_TILE_KS(MAPS, DVT, KS)                                                                                                  \
   do {                                                                                                                           \
     if (head_rows)                                                                                                               \
-      hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, true>), grid, dim3(64), lds, stream, (bf16*)out, ldo, (const bf16*)q, ldq, \
+      hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, true, KS>), grid, dim3(64), lds, stream, (bf16*)out, ldo, (const bf16*)q, ldq, \
                          q_head, (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, tiles, max_blocks,   \
                          num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, part);  \
     else                                                                                                                         \
-      hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, false>), grid, dim3(64 * nw), lds, stream, (bf16*)out, ldo,              \
+      hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, false, KS>), grid, dim3(64 * nw), lds, stream, (bf16*)out, ldo,              \
                          (const bf16*)q, ldq, q_head, (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, \
                          tiles, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps,  \
                          gate, ldg, part);                                                                                       \
+  } while (0)
+  // (a map's whole key row in flight when it is long and the registers allow: one wait per block instead of four)
+#define DLIA_TILE(MAPS, DVT)                                            \
+  do {                                                                  \
+    if (MAPS == 1 && d > 128) DLIA_TILE_KS(MAPS, DVT, (MAPS == 1 ? 16 : 4)); \
+    else DLIA_TILE_KS(MAPS, DVT, 4);                                   \
   } while (0)
   if (maps == 2) {
     if (dvt == 4) DLIA_TILE(2, 4); else if (dvt == 8) DLIA_TILE(2, 8); else if (dvt == 16) DLIA_TILE(2, 16); else DLIA_TILE(2, 32);
@@ -859,5 +865,6 @@ extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq,
                          post, eps, gate, ldg);
   }
 #undef DLIA_TILE
+#undef DLIA_TILE_KS
   return 0;
 }
