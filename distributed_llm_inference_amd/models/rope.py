@@ -35,9 +35,13 @@ def scaled_inv_frequencies(d: int, theta: float, rs) -> torch.Tensor:
         if rs.truncate:
             low, high = math.floor(low), math.ceil(high)
         low, high = max(low, 0), min(high, d - 1)
-        if low == high:
-            high += 0.001
-        ramp = ((torch.arange(d // 2, dtype=torch.float64) - low) / (high - low)).clamp(0, 1)
+        if rs.ramp_floor:
+            width = max(high - low, 0.001)
+        else:
+            if low == high:
+                high += 0.001
+            width = high - low
+        ramp = ((torch.arange(d // 2, dtype=torch.float64) - low) / width).clamp(0, 1)
         inv = (inv / rs.factor) * ramp + inv * (1 - ramp)
     elif rs is not None:
         # Llama-3.1 frequency-dependent rescale: long wavelengths are divided by `factor`,

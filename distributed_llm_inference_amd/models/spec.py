@@ -35,6 +35,9 @@ class RopeScaling:
     beta_slow: float = 1.0
     attention_factor: Optional[float] = None
     truncate: bool = True
+    # yarn: the ramp's width is max(high - low, 0.001) (a band that the clamps turn inside out counts as empty) instead of
+    # high - low with only the equal case widened
+    ramp_floor: bool = False
 
 
 def distance_bucket(n: int, rows: int, far: int) -> int:
@@ -449,7 +452,7 @@ class ModelSpec:
             sc, scaling = rot.get("scaling"), None
             if sc:
                 scaling = RopeScaling(factor=float(sc["factor"]), rope_type="yarn", beta_fast=float(sc["fast"]), beta_slow=float(sc["slow"]),
-                                      original_max_position_embeddings=int(sc["original"]))
+                                      original_max_position_embeddings=int(sc["original"]), ramp_floor=True)
             return dict(rope_dims=int(rot["dims"]), rope_base=float(rot["base"]), rope_interleaved=interleaved, rope_scaling=scaling)
 
         layers = []
@@ -868,7 +871,8 @@ def tezesun_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
     dm = max(2, head_dim // 2)
     att = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=dm, vdim=head_dim, window=window, keep_first=keep_first,
                     scale=dm ** -0.5, softcap=30.0, maps=2, diff=0.5, out_gate=True, rope_dims=dm, rope_base=1000000.0, rope_interleaved=True,
-                    rope_scaling=RopeScaling(factor=4.0, rope_type="yarn", beta_fast=32.0, beta_slow=1.0, original_max_position_embeddings=4096),
+                    rope_scaling=RopeScaling(factor=4.0, rope_type="yarn", beta_fast=32.0, beta_slow=1.0, original_max_position_embeddings=4096,
+                                             ramp_floor=True),
                     ff=ff, ff_kind="xielu")
     lat = LayerSpec("latent_attention", heads=heads, kv_heads=1, dim=head_dim, vdim=head_dim, scale=(head_dim + rot_dim) ** -0.5,
                     q_rank=q_rank or max(8, width // 2), kv_rank=kv_rank or max(8, width // 8), rot_dim=rot_dim, rope_dims=rot_dim,

@@ -39,10 +39,12 @@ def test_partial_rotation_and_scaled_frequencies(interleaved, dims, D):
     from distributed_llm_inference_amd.models.rope import rope_table
     from distributed_llm_inference_amd.models.spec import RopeScaling
     from distributed_llm_inference_amd.ops import reference as R
-    for sc in (None, {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}, {"factor": 6.0, "original": 1000, "fast": 24.0, "slow": 1.5}):
+    # (the last one: a band that lies beyond the rotated entries, which the clamps turn inside out: no frequency is rescaled)
+    for sc in (None, {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}, {"factor": 6.0, "original": 1000, "fast": 24.0, "slow": 1.5},
+               {"factor": 3.0, "original": 10 ** 7, "fast": 16.0, "slow": 2.0}):
         rot = {"dims": dims, "base": 100.0, **({"scaling": sc} if sc else {})}
         rs = RopeScaling(factor=sc["factor"], rope_type="yarn", beta_fast=sc["fast"], beta_slow=sc["slow"],
-                         original_max_position_embeddings=sc["original"]) if sc else None
+                         original_max_position_embeddings=sc["original"], ramp_floor=True) if sc else None
         cos, sin = rope_table(dims, 100.0, rs, 50)
         rc, rsn = O.rope_angles(rot, 50)
         close(cos, rc, 1e-6)
