@@ -324,3 +324,14 @@ def test_trace_run_executable(models, tmp_path):
     check(got[0], ra[[0, 32]], "fp32")
     check(got[1], ra[[33]], "fp32")
     check(got[2], np.stack([ra[39], rb[8]]), "fp32")
+
+
+def test_generate_command(capsys):
+    """The command line's `generate` on a built-in Tezesun stack (CPU: torch executor)."""
+    import json
+    from distributed_llm_inference_amd.serving import cli
+    rc = cli.main(["generate", "Hello", "--model", "tiny-tezesun-test", "--device", "cpu", "--backend", "torch",
+                   "--max-tokens", "5", "--temperature", "0", "--max-seq-len", "128"])
+    assert rc == 0
+    d = json.loads(capsys.readouterr().out)
+    assert d["status"] == "success" and d["tokens_generated"] <= 5 and d["prompt"] == "Hello"
