@@ -390,6 +390,24 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
           s[a][1] = mfma16(ak[a][u][1], bq, s[a][1]);
         }
     }
+    // Up to 16 accumulator tiles: the value fragments of the block's first VB tiles are asked for now, so that their way from
+    // memory overlaps the softmax. (With more accumulators the registers do not hold them as well: fragment by fragment then.)
+    constexpr bool AHEAD = MAPS * DVT <= 16;
+    constexpr int VB = DVT > 8 ? 8 : DVT;
+    const bf16* vbase = vt + ((long)blk * G + g) * dv * kParBlock + (long)r16 * kParBlock + kq * 4;
+    u32x4 av[VB];
+    auto load_values = [&](int c0) {
+#pragma unroll
+      for (int j = 0; j < VB; ++j) {
+        av[j] = zero;
+        if ((c0 + j) * 16 + r16 < dv) {
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(vbase + (long)(c0 + j) * 16 * kParBlock);
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(vbase + (long)(c0 + j) * 16 * kParBlock + 16);
+          av[j] = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+      }
+    };
+    if constexpr (AHEAD) load_values(0);
     u32x4 pf[MAPS];
 #pragma unroll
     for (int a = 0; a < MAPS; ++a) {
@@ -422,19 +440,31 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
       for (int c = 0; c < DVT; ++c) o[a][c] *= corr;
       pf[a] = pack8(p);
     }
-    const bf16* vbase = vt + ((long)blk * G + g) * dv * kParBlock;
+    if constexpr (AHEAD) {
 #pragma unroll
-    for (int c = 0; c < DVT; ++c) {
-      if (c * 16 >= dv) break;
-      const int row = c * 16 + r16;
-      u32x4 av = zero;
-      if (row < dv) {
-        const u32x2 lo = *reinterpret_cast<const u32x2*>(vbase + (long)row * kParBlock + kq * 4);
-        const u32x2 hi = *reinterpret_cast<const u32x2*>(vbase + (long)row * kParBlock + 16 + kq * 4);
-        av = u32x4{lo.x, lo.y, hi.x, hi.y};
+      for (int c0 = 0; c0 < DVT; c0 += VB) {
+        if (c0 * 16 >= dv) break;
+        if (c0 > 0) load_values(c0);
+#pragma unroll
+        for (int j = 0; j < VB; ++j) {
+          if ((c0 + j) * 16 >= dv) break;
+#pragma unroll
+          for (int a = 0; a < MAPS; ++a) o[a][c0 + j] = mfma16(av[j], pf[a], o[a][c0 + j]);
+        }
       }
+    } else {
 #pragma unroll
-      for (int a = 0; a < MAPS; ++a) o[a][c] = mfma16(av, pf[a], o[a][c]);
+      for (int c = 0; c < DVT; ++c) {
+        if (c * 16 >= dv) break;
+        u32x4 v1 = zero;
+        if (c * 16 + r16 < dv) {
+          const u32x2 lo = *reinterpret_cast<const u32x2*>(vbase + (long)c * 16 * kParBlock);
+          const u32x2 hi = *reinterpret_cast<const u32x2*>(vbase + (long)c * 16 * kParBlock + 16);
+          v1 = u32x4{lo.x, lo.y, hi.x, hi.y};
+        }
+#pragma unroll
+        for (int a = 0; a < MAPS; ++a) o[a][c] = mfma16(v1, pf[a], o[a][c]);
+      }
     }
   }
   float inv[MAPS];
