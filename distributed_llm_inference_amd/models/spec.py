@@ -85,9 +85,15 @@ class LayerSpec:
     `rope_dims` > 0: the first rope_dims entries of every q / k vector are rotated by position, frequencies
     `rope_base`^(-2i / rope_dims), pairs (2i, 2i + 1) when `rope_interleaved` else (i, i + rope_dims / 2), rescaled
     by `rope_scaling` when given.
+    `proj_bias`: the q, k, v and output projections have biases. `qk_norm`: q and k are RMS-normed over the WHOLE projection
+    (all heads at once, a learned weight per entry) before the rotation. `v_norm`: every head's value is divided by its root
+    mean square (no weight) before it is cached. `head_mix`: the heads' scaled scores are mixed by a learned [heads, heads]
+    matrix before mask and softmax, s_h <- sum_g M[h, g] s_g. `chunk` > 0: a query at i sees the keys j <= i of its own
+    chunk only, floor(i / chunk) = floor(j / chunk), chunks counted from the sequence's position 0.
+    ``parallel`` with `branch_scales` (a, b): the branches' outputs are added as a * left + b * right (no norms, no average).
     The feed-forward sublayer is `ff_kind`: ``gated_gelu`` (gelu_tanh(gate) * up, biases), ``gelu`` (up, exact
-    GELU, down; no biases), ``xielu`` (up, a two-sided quadratic / exponential unit with two learned numbers, down) or
-    ``moe`` (`moe` says how tokens are routed to its experts)."""
+    GELU, down; no biases), ``xielu`` (up, a two-sided quadratic / exponential unit with two learned numbers, down),
+    ``relu2`` (up, the square of relu, down; biases) or ``moe`` (`moe` says how tokens are routed to its experts)."""
     kind: str                       # "attention" | "delta" | "general_delta" | "mlstm" | "parallel" | "rglru" | "latent_attention"
     heads: int
     kv_heads: int
@@ -124,6 +130,12 @@ class LayerSpec:
     rot_dim: int = 0
     rec_width: int = 0
     blocks: int = 1
+    proj_bias: bool = False
+    qk_norm: bool = False
+    v_norm: bool = False
+    head_mix: bool = False
+    chunk: int = 0
+    branch_scales: tuple = ()
 
     @property
     def group(self) -> int:
@@ -172,9 +184,11 @@ class LayerSpec:
 
     def ff_param_count(self, width: int) -> int:
         if self.moe is not None:
-            return self.moe.experts * (3 * width * self.moe.ff + width)
+            return self.moe.experts * (3 * width * self.moe.ff + width) + 3 * width * self.moe.shared_ff
         if self.ff_kind in ("gelu", "xielu"):
             return 2 * width * self.ff
+        if self.ff_kind == "relu2":
+            return 2 * width * self.ff + self.ff + width
         return 3 * width * self.ff + 2 * self.ff + width if self.ff else 0
 
 
@@ -185,7 +199,14 @@ class MoeSpec:
     size; a block is ranked by its best two scores added up, and the choice is made among the experts of the
     `keep` best blocks. The outputs of the chosen experts are summed with weights score / (sum of the chosen
     scores) * `scale`. An
-    expert computes down(g sigmoid(1.702 g) (u + 1)) with g = min(gate(x), limit), u = clamp(up(x), +-limit)."""
+    expert computes down(g sigmoid(1.702 g) (u + 1)) with g = min(gate(x), limit), u = clamp(up(x), +-limit).
+    Switches: `score` ``softmax``: scores are the softmax of the logits over all router outputs. `correction`: the CHOICE
+    (of groups and of experts) goes by score + a learned number per router output, the weights by the score alone.
+    `group_rank`: how many of a block's best choice scores are added up to rank it (1: its best). `renorm` off: the weights
+    are the chosen scores times `scale`, not divided by their sum. `identity`: the router has that many outputs more than
+    there are experts; choosing one of them returns the token's input itself (times the weight); they count as experts for
+    the groups. `shared_ff` > 0: one more expert of that width runs for every token and is added unweighted. `act`
+    ``silu``: an expert computes down(silu(gate(x)) * up(x)), no limits."""
     experts: int
     top: int
     ff: int
@@ -193,12 +214,24 @@ class MoeSpec:
     keep: int = 1
     scale: float = 1.0
     limit: float = 7.0
+    score: str = "sigmoid"
+    correction: bool = False
+    group_rank: int = 2
+    renorm: bool = True
+    identity: int = 0
+    shared_ff: int = 0
+    act: str = "swish_lim"
+
+    @property
+    def outputs(self) -> int:
+        """Outputs of the router: the experts and the identity experts."""
+        return self.experts + self.identity
 
 
 @dataclass(frozen=True)
 class ModelSpec:
     name: str
-    family: str                     # "llama" | "gpt2" | "letarax" | "nufapel" | "tezesun"
+    family: str                     # "llama" | "gpt2" | "letarax" | "nufapel" | "tezesun" | "zovozen"
     num_layers: int
     hidden_size: int
     num_heads: int
@@ -243,6 +276,9 @@ class ModelSpec:
     layer_scale: bool = False
     token_shift: bool = False
     logit_scale: float = 1.0                 # the logits are multiplied by it
+    # `post_norm`: the sublayers read the residual stream itself and a plain-weight RMS norm sits on their OUTPUT only:
+    # x += norm1(mixer(x)); x += norm2(ff(x))
+    post_norm: bool = False
 
     @property
     def is_hybrid(self) -> bool:
@@ -497,6 +533,92 @@ class ModelSpec:
             layer_specs=tuple(layers), parallel_block=True, layer_scale=True, token_shift=True,
             logit_scale=float(cfg.get("logit_scale", 1.0)))
 
+    @staticmethod
+    def from_zovozen_config(cfg: Dict[str, Any], name: str = "") -> "ModelSpec":
+        """Zovozen: every layer is a ``parallel`` pair reading the residual stream itself, with RMS norms on the sublayers'
+        outputs only. mixer.left: attention (heads, kv_heads, dim, vdim, scale, mask.size = chunk, rot.dims / base /
+        scaling.factor) with biased projections, whole-projection q / k norms, unit values, head temperatures, mixed heads,
+        learned sinks and an output gate; mixer.right: matrix memory (heads, dim, vdim, gate_cap); left_scale / right_scale
+        weigh their sum. ``mlp``: null, ``dense`` (ff; squared relu, biases) or ``moe`` (expert.ff, router.experts / top /
+        identity / groups.count / groups.keep, shared.ff). The head is the embedding table. Keys a config leaves out switch
+        their mechanism off."""
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m, mlp = l["mixer"], l.get("mlp")
+            if l["type"] != "parallel":
+                raise ValueError(f"layer {i}: unknown mixer type {l['type']!r}")
+            ffkw: Dict[str, Any] = dict(ff=0, ff_kind="relu2")
+            if mlp is not None and mlp.get("kind", "dense") == "dense":
+                ffkw = dict(ff=int(mlp["ff"]), ff_kind="relu2")
+            elif mlp is not None and mlp["kind"] == "moe":
+                r, g = mlp["router"], (mlp["router"].get("groups") or {})
+                moe = MoeSpec(experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]), groups=int(g.get("count", 1)),
+                              keep=int(g.get("keep", g.get("count", 1))), scale=1.0, limit=0.0, score="softmax", correction=True,
+                              group_rank=1, renorm=False, identity=int(r.get("identity") or 0),
+                              shared_ff=int((mlp.get("shared") or {}).get("ff") or 0), act="silu")
+                if moe.outputs % moe.groups or not 1 <= moe.keep <= moe.groups or not 1 <= moe.top <= moe.keep * (moe.outputs // moe.groups):
+                    raise ValueError(f"layer {i}: {moe.outputs} router outputs in {moe.groups} groups, {moe.keep} kept, {moe.top} chosen")
+                ffkw = dict(ff=0, ff_kind="moe", moe=moe)
+            elif mlp is not None:
+                raise ValueError(f"layer {i}: feed-forward kind {mlp.get('kind')!r} is not supported (dense and moe are)")
+            a, b = m["left"], m["right"]
+            if int(a["heads"]) % int(a["kv_heads"]):
+                raise ValueError(f"layer {i}: {a['heads']} heads over {a['kv_heads']} key / value heads")
+            rot = a.get("rot") or {}
+            rp: Dict[str, Any] = {}
+            if int(rot.get("dims") or 0):
+                if int(rot["dims"]) % 2 or int(rot["dims"]) > int(a["dim"]):
+                    raise ValueError(f"layer {i}: {rot['dims']} rotated entries of {a['dim']}")
+                f = float((rot.get("scaling") or {}).get("factor") or 1.0)
+                rp = dict(rope_dims=int(rot["dims"]), rope_base=float(rot["base"]), rope_interleaved=False,
+                          rope_scaling=RopeScaling(factor=f, rope_type="linear") if f != 1.0 else None)
+            left = LayerSpec("attention", heads=int(a["heads"]), kv_heads=int(a["kv_heads"]), dim=int(a["dim"]), vdim=int(a["vdim"]),
+                             scale=float(a["scale"]), sink=True, sink_learned=True, head_temp=True, out_gate=True, proj_bias=True,
+                             qk_norm=True, v_norm=True, head_mix=True, chunk=int((a.get("mask") or {}).get("size") or 0), **rp)
+            right = LayerSpec("mlstm", heads=int(b["heads"]), kv_heads=int(b["heads"]), dim=int(b["dim"]), vdim=int(b["vdim"]),
+                              gate_cap=float(b["gate_cap"]), scale=float(b["dim"]) ** -0.5)
+            layers.append(LayerSpec("parallel", heads=left.heads, kv_heads=left.kv_heads, dim=left.dim, vdim=left.vdim,
+                                    branches=(left, right), branch_scales=(float(m.get("left_scale", 1.0)), float(m.get("right_scale", 1.0))),
+                                    **ffkw))
+        if not layers:
+            raise ValueError("a model needs at least one layer")
+        heads = [b for l in layers for b in l.branches]
+        return ModelSpec(
+            name=name or "zovozen", family="zovozen", num_layers=len(layers), hidden_size=int(cfg["width"]),
+            num_heads=max(l.heads for l in heads), num_kv_heads=max(l.kv_heads for l in heads),
+            head_dim=max(max(l.dim, l.vdim) for l in heads),
+            intermediate_size=max(max(l.ff, l.moe.ff if l.moe else 0, l.moe.shared_ff if l.moe else 0) for l in layers),
+            vocab_size=int(cfg["vocab"]), max_position=1 << 30, norm_eps=float(cfg["norm"]["eps"]), tie_embeddings=True,
+            bos_token_id=cfg.get("bos_token_id"), eos_token_id=_scalar_eos(cfg.get("eos_token_id")), hf_type="zovozen",
+            layer_specs=tuple(layers), post_norm=True)
+
+    def zovozen_config(self) -> Dict[str, Any]:
+        """The inverse of `from_zovozen_config`."""
+        out = []
+        for l in self.layer_specs:
+            a, b = l.branches
+            left: Dict[str, Any] = {"heads": a.heads, "kv_heads": a.kv_heads, "dim": a.dim, "vdim": a.vdim, "scale": a.scale}
+            if a.chunk:
+                left["mask"] = {"size": a.chunk}
+            if a.rope_dims:
+                left["rot"] = {"base": a.rope_base, "dims": a.rope_dims}
+                if a.rope_scaling is not None:
+                    left["rot"]["scaling"] = {"factor": a.rope_scaling.factor}
+            m = {"left": left, "right": {"heads": b.heads, "dim": b.dim, "vdim": b.vdim, "gate_cap": b.gate_cap},
+                 "left_scale": l.branch_scales[0], "right_scale": l.branch_scales[1]}
+            if l.moe is not None:
+                e = l.moe
+                mlp: Optional[Dict[str, Any]] = {"kind": "moe", "expert": {"ff": e.ff},
+                                                 "router": {"experts": e.experts, "top": e.top, "identity": e.identity,
+                                                            "groups": {"count": e.groups, "keep": e.keep}}}
+                if e.shared_ff:
+                    mlp["shared"] = {"ff": e.shared_ff}
+            else:
+                mlp = {"kind": "dense", "ff": l.ff} if l.ff else None
+            out.append({"type": "parallel", "mixer": m, "mlp": mlp})
+        return {"architecture": "Zovozen", "layers": out, "norm": {"eps": self.norm_eps}, "vocab": self.vocab_size,
+                "width": self.hidden_size, "bos_token_id": self.bos_token_id, "eos_token_id": self.eos_token_id}
+
     def tezesun_config(self) -> Dict[str, Any]:
         """The inverse of `from_tezesun_config`."""
         def rot_of(l):
@@ -579,6 +701,8 @@ class ModelSpec:
             return ModelSpec.from_nufapel_config(cfg, name=name)
         if cfg.get("architecture") == "Tezesun":
             return ModelSpec.from_tezesun_config(cfg, name=name)
+        if cfg.get("architecture") == "Zovozen":
+            return ModelSpec.from_zovozen_config(cfg, name=name)
         if mt == "gpt2" or any("GPT2" in a for a in archs):
             if cfg.get("activation_function", "gelu_new") != "gelu_new" or cfg.get("scale_attn_by_inverse_layer_idx"):
                 raise ValueError("GPT-2 variants other than gelu_new MLPs with plain 1/sqrt(d) attention scaling are not supported")
@@ -710,7 +834,7 @@ class ModelSpec:
     def hf_config(self) -> Dict[str, Any]:
         """The inverse of `from_hf_config`: a config.json dict for this spec."""
         if self.is_hybrid:
-            return {"nufapel": self.nufapel_config, "tezesun": self.tezesun_config}.get(self.family, self.letarax_config)()
+            return {"nufapel": self.nufapel_config, "tezesun": self.tezesun_config, "zovozen": self.zovozen_config}.get(self.family, self.letarax_config)()
         if self.is_gpt2:
             return {
                 "model_type": "gpt2", "architectures": ["GPT2LMHeadModel"],
@@ -885,6 +1009,31 @@ def tezesun_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
                      layer_scale=True, token_shift=True, logit_scale=1.5)
 
 
+def zovozen_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int, ff: int, num_layers: int, vocab_size: int = 32000,
+                 pattern: str = "md", experts: int = 8, top: int = 2, identity: int = 2, groups: int = 2, keep: int = 1, chunk: int = 1024,
+                 vdim: int = 0, rot_dims: int = 0, mem_heads: int = 0, shared: bool = True) -> ModelSpec:
+    """A Zovozen stack from a few numbers: every layer is attention (biased projections, whole-projection q / k norms, unit
+    values, half-rotated heads with linearly rescaled frequencies, head temperatures, mixed heads, learned sinks, chunked
+    mask, output gate) beside a matrix memory of `mem_heads` heads (half as many by default); `pattern` repeats over the
+    layers' feed-forwards: 'd' dense squared-relu of `ff`, 'm' routed (`experts` experts of ff / 4 plus `identity` identity
+    experts in `groups` groups, `top` chosen from `keep` groups, a shared expert of ff / 2), 'n' none."""
+    moe = MoeSpec(experts=experts, top=top, ff=max(8, ff // 4), groups=groups, keep=keep, scale=1.0, limit=0.0, score="softmax",
+                  correction=True, group_rank=1, renorm=False, identity=identity, shared_ff=max(8, ff // 2) if shared else 0, act="silu")
+    rd = rot_dims or max(2, head_dim // 2)
+    left = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=vdim or head_dim, scale=head_dim ** -0.5, sink=True,
+                     sink_learned=True, head_temp=True, out_gate=True, proj_bias=True, qk_norm=True, v_norm=True, head_mix=True, chunk=chunk,
+                     rope_dims=rd, rope_base=250000.0, rope_scaling=RopeScaling(factor=4.0, rope_type="linear"))
+    mh = mem_heads or max(1, heads // 2)
+    right = LayerSpec("mlstm", heads=mh, kv_heads=mh, dim=head_dim, vdim=vdim or head_dim, gate_cap=15.0, scale=head_dim ** -0.5)
+    par = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=vdim or head_dim, branches=(left, right), branch_scales=(0.75, 0.6))
+    kinds = {"d": LayerSpec("parallel", ff=ff, ff_kind="relu2", **par), "m": LayerSpec("parallel", ff=0, ff_kind="moe", moe=moe, **par),
+             "n": LayerSpec("parallel", ff=0, ff_kind="relu2", **par)}
+    layers = tuple(kinds[pattern[i % len(pattern)]] for i in range(num_layers))
+    return ModelSpec(name=name, family="zovozen", num_layers=num_layers, hidden_size=width, num_heads=heads, num_kv_heads=kv_heads,
+                     head_dim=max(head_dim, vdim), intermediate_size=ff, vocab_size=vocab_size, max_position=1 << 30, norm_eps=1e-5,
+                     tie_embeddings=True, bos_token_id=1, eos_token_id=2, hf_type="zovozen", layer_specs=layers, post_norm=True)
+
+
 # Letarax stacks of the sizes of the Llama benchmark shapes (random weights; `bench.py --hybrid-compare` runs them)
 BUILTIN_SPECS["letarax-1b-like"] = letarax_spec("letarax-1b-like", 2048, 16, 4, 128, 8192, 8, 1024)
 BUILTIN_SPECS["letarax-8b-like"] = letarax_spec("letarax-8b-like", 4096, 32, 8, 128, 14336, 4, 2048)
@@ -894,6 +1043,9 @@ BUILTIN_SPECS["nufapel-8b-like"] = nufapel_spec("nufapel-8b-like", 4096, 32, 8, 
 # Tezesun stacks of the same sizes (`bench.py --parallel-compare` runs them beside the Letarax stacks)
 BUILTIN_SPECS["tezesun-1b-like"] = tezesun_spec("tezesun-1b-like", 2048, 16, 4, 128, 8192, 8, window=1024, kv_rank=448, rot_dim=64, q_rank=1024)
 BUILTIN_SPECS["tezesun-8b-like"] = tezesun_spec("tezesun-8b-like", 4096, 32, 8, 128, 14336, 4, window=2048, kv_rank=448, rot_dim=64, q_rank=1536)
+# Zovozen stacks of the same sizes (`bench.py --postnorm-compare` runs them beside the Nufapel stacks)
+BUILTIN_SPECS["zovozen-1b-like"] = zovozen_spec("zovozen-1b-like", 2048, 16, 4, 128, 8192, 8, chunk=1024)
+BUILTIN_SPECS["zovozen-8b-like"] = zovozen_spec("zovozen-8b-like", 4096, 32, 8, 128, 14336, 4, chunk=2048)
 
 
 def _register_test_models():
@@ -917,6 +1069,10 @@ def _register_test_models():
                                                       q_rank=24, kv_rank=20, rot_dim=8, keep_first=3)
     BUILTIN_SPECS["tiny-tezesun-gpu-test"] = tezesun_spec("tiny-tezesun-gpu-test", 128, 4, 2, 32, 256, 4, window=36, vocab_size=320, blocks=2,
                                                           q_rank=48, kv_rank=40, rot_dim=16, keep_first=5)
+    BUILTIN_SPECS["tiny-zovozen-test"] = zovozen_spec("tiny-zovozen-test", 64, 4, 2, 16, 96, 3, vocab_size=320, pattern="dmn", experts=6,
+                                                      identity=2, groups=4, keep=2, chunk=20, vdim=24, rot_dims=8)
+    BUILTIN_SPECS["tiny-zovozen-gpu-test"] = zovozen_spec("tiny-zovozen-gpu-test", 128, 4, 2, 32, 256, 4, vocab_size=320, pattern="mdm",
+                                                          experts=6, identity=2, groups=2, keep=1, chunk=40, vdim=48, rot_dims=16)
     BUILTIN_SPECS["tiny-gpt2-gpu-test"] = tiny_spec(
         "gpt2", name="tiny-gpt2-gpu-test", hidden_size=256, num_heads=4, num_kv_heads=4, head_dim=64,
         intermediate_size=1024, vocab_size=333, num_layers=4)

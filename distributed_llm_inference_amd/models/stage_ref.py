@@ -347,10 +347,100 @@ class RefStage:
             self.layer_outputs.append(h)
         return h
 
+    # -- hybrid stacks whose sublayers read the stream itself, with RMS norms on their outputs only ------------------
+    def _postnorm_layers(self, batch: StepBatch, h: torch.Tensor) -> torch.Tensor:
+        """x <- x + norm1(a * left(x) + b * right(x)); x <- x + norm2(ff(x)) for every layer: attention (whole-projection
+        q / k norms, partial rotation, unit values, head temperatures, mixed heads, chunked mask, learned sink, output gate)
+        beside a matrix memory; dense squared-relu or routed feed-forward (softmax scores, corrected choice, identity and
+        shared experts). Norms, rotations, scores, routers, gates of the recurrence, its state and the residual sum are fp32
+        whatever the dtype."""
+        from .rope import rope_table
+        spec, dt, eps, w = self.spec, self.dtype, self.spec.norm_eps, self.w
+        T, dev = h.shape[0], self.device
+        F = torch.nn.functional
+        lin = lambda x, m, b=None: R.gemm(x.to(dt), m, b, None, 1 if b is not None else 0)
+        rnd = lambda x: x.to(dt).float()
+        seqs, t0 = [], 0
+        for slot, qlen, ctx in zip(batch.slots, batch.q_lens, batch.ctx_lens):
+            if qlen > 0 and ctx == 0:
+                self.cache.pop(slot, None)            # a sequence's first tokens: whatever the slot held before is void
+            if qlen > 0:
+                seqs.append((slot, t0, qlen, ctx))
+            t0 += qlen
+        pos = torch.tensor([c + i for c, q in zip(batch.ctx_lens, batch.q_lens) for i in range(q)], dtype=torch.long, device=dev)
+        far = int(pos.max()) + 1 if T else 1
+        ones = lambda n: torch.ones(n, device=dev)
+        self.layer_outputs = []
+        for li, l in enumerate(w.layers):
+            ls = spec.layer_specs[self.plan.layers[li]]
+            a, b = ls.branches
+            sizes = [a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim, a.heads * a.vdim, b.heads * b.dim, b.heads * b.dim,
+                     b.heads * b.vdim, b.heads * b.vdim, b.heads, b.heads]
+            z = lin(h, l["w_in"])
+            q, k, v, gl, rq, rk, rv, rg, ri_, rf_ = torch.split(z, sizes, dim=1)
+            bq, bk, bv = torch.split(l["b_qkv"].float(), sizes[:3])
+            q, k, v = q + bq, k + bk, v + bv
+            if a.qk_norm:
+                q, k = R.rmsnorm(q, l["q_norm_w"], eps), R.rmsnorm(k, l["k_norm_w"], eps)
+            q, k, v = q.reshape(T, a.heads, a.dim), k.reshape(T, a.kv_heads, a.dim), v.reshape(T, a.kv_heads, a.vdim)
+            if a.rope_dims:
+                cos, sin = rope_table(a.rope_dims, a.rope_base, a.rope_scaling, far, dev)
+                q, k = R.rope_partial(q, cos, sin, pos, a.rope_interleaved), R.rope_partial(k, cos, sin, pos, a.rope_interleaved)
+            if a.v_norm:
+                v = R.rmsnorm(v, ones(a.vdim), eps)
+            left = torch.empty(T, a.heads, a.vdim, dtype=torch.float32, device=dev)
+            right = torch.empty(T, b.heads, b.vdim, dtype=torch.float32, device=dev)
+            li_ = b.gate_cap * torch.tanh((ri_ + l["b_if"][:b.heads].float()) / b.gate_cap)
+            lf_ = F.logsigmoid(b.gate_cap * torch.tanh((rf_ + l["b_if"][b.heads:].float()) / b.gate_cap))
+            for slot, s0, qlen, ctx in seqs:
+                sta, stb = self._slot_cache(slot)[li]
+                sl = slice(s0, s0 + qlen)
+                assert sta[0].shape[0] >= ctx, f"slot {slot}: cache has {sta[0].shape[0]} tokens, step says {ctx}"
+                sta[0] = torch.cat([sta[0][:ctx], k[sl].to(dt)])
+                sta[1] = torch.cat([sta[1][:ctx], v[sl].to(dt)])
+                left[sl] = R.attention(q[sl].to(dt), sta[0], sta[1], ctx, a.scale, sink=a.sink, temp=l["temp"] if a.head_temp else None,
+                                       sink_logit=l["sink"] if a.sink_learned else None, chunk=a.chunk,
+                                       head_mix=l["talk"] if a.head_mix else None)
+                right[sl], stb[0], stb[1], stb[2] = R.matrix_memory(
+                    rq[sl].reshape(qlen, b.heads, b.dim) * b.scale, rk[sl].reshape(qlen, b.heads, b.dim),
+                    rv[sl].reshape(qlen, b.heads, b.vdim), li_[sl], lf_[sl], stb[0], stb[1], stb[2])
+            left = left.reshape(T, -1) * torch.sigmoid(gl)
+            right = R.rmsnorm(right, ones(b.vdim), eps).reshape(T, -1) * l["o_norm_w"].float() * torch.sigmoid(rg)
+            y = ls.branch_scales[0] * lin(left, l["w_o"], l["b_o"]) + ls.branch_scales[1] * lin(right, l["w_o_r"])
+            h = h + R.rmsnorm(y, l["ln1_w"], eps)
+            if ls.has_ff:
+                if ls.moe is None:
+                    y = lin(rnd(torch.relu(lin(h, l["w_up"], l["b_up"])) ** 2), l["w_down"], l["b_down"])
+                else:
+                    e = ls.moe
+                    glu = lambda x, g_, u_, d_: lin(rnd(F.silu(lin(x, g_)) * lin(x, u_)), d_)
+                    idx, wts = R.moe_route(torch.softmax(lin(h, l["w_router"]), dim=-1), e.top, e.groups, e.keep, e.scale,
+                                           correction=l["correction"], group_rank=e.group_rank, renorm=e.renorm)
+                    y = torch.zeros_like(h)
+                    for ex in range(e.outputs):
+                        rows, col = (idx == ex).nonzero(as_tuple=True)
+                        if rows.numel() == 0:
+                            continue
+                        out = h[rows] if ex >= e.experts else glu(h[rows], l["w_gate_e"][ex], l["w_up_e"][ex], l["w_down_e"][ex])
+                        y.index_add_(0, rows, out * wts[rows, col].unsqueeze(1))
+                    if e.shared_ff:
+                        y = y + glu(h, l["w_gate_s"], l["w_up_s"], l["w_down_s"])
+                h = h + R.rmsnorm(y, l["ln2_w"], eps)
+            self.layer_outputs.append(h)
+        return h
+
     def _forward_hybrid(self, batch: StepBatch, x: torch.Tensor) -> torch.Tensor:
         T = batch.num_tokens
         ids = torch.as_tensor(x).to(self.device).long().reshape(-1)
         assert ids.numel() == T, f"expected {T} token ids, got {ids.numel()}"
+        if self.spec.post_norm:
+            h = self._postnorm_layers(batch, self.w.embed[ids].float())
+            self.last_hidden = h
+            rows = self._out_rows(batch)
+            if not rows:
+                return torch.empty(0, self.spec.vocab_size, dtype=torch.float32, device=self.device)
+            hn = R.rmsnorm(h[rows], self.w.final_norm_w, self.spec.norm_eps)
+            return R.gemm(hn.to(self.dtype), self.w.lm_head).float()
         if self.spec.parallel_block:
             h = self._parallel_layers(batch, self.w.embed[ids].float())
             self.last_hidden = h

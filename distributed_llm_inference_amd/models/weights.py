@@ -340,6 +340,122 @@ def _random_tezesun_weights(spec: ModelSpec, plan: StagePlan, seed: int, device,
         w.layers.append(l)
     return w
 
+# ---- Zovozen: checkpoint names <-> the logical layout ----------------------------------------------------------------
+# Per layer: ln1_w / ln2_w (the norms on the sublayers' outputs);
+#   mixer:  w_in = left q | k | v | g, right q | k | v | g | i | f (one GEMM), b_qkv (left q | k | v), q_norm_w, k_norm_w,
+#           talk [heads, heads], temp, sink, w_o / b_o (left); b_if, o_norm_w, w_o_r (right)
+#   dense:  w_up / b_up, w_down / b_down
+#   moe:    w_router [experts + identity, H], correction, w_gate_e / w_up_e [E, ff, H], w_down_e [E, H, ff],
+#           shared expert w_gate_s / w_up_s / w_down_s
+def _zovozen_layer_names(ls, p: str) -> Dict[str, object]:
+    """logical name -> checkpoint name, or a tuple of names that are concatenated (dim 0), or a list that is stacked (experts)."""
+    m, f = p + "mix.", p + "mlp."
+    n: Dict[str, object] = {
+        "ln1_w": p + "norm1", "w_in": tuple(m + x for x in _PAR_IN), "b_qkv": (m + "left.q.b", m + "left.k.b", m + "left.v.b"),
+        "q_norm_w": m + "left.q.norm", "k_norm_w": m + "left.k.norm", "talk": m + "left.talk", "temp": m + "left.temp",
+        "sink": m + "left.sink", "w_o": m + "left.o", "b_o": m + "left.o.b", "b_if": (m + "right.i.b", m + "right.f.b"),
+        "o_norm_w": m + "right.norm", "w_o_r": m + "right.o"}
+    if ls.has_ff:
+        n["ln2_w"] = p + "norm2"
+        if ls.moe is not None:
+            n.update({"w_router": f + "router", "correction": f + "correction"})
+            for x in ("gate", "up", "down"):
+                n[f"w_{x}_e"] = [f"{f}e{e}.{x}" for e in range(ls.moe.experts)]
+                if ls.moe.shared_ff:
+                    n[f"w_{x}_s"] = f"{f}shared.{x}"
+        else:
+            n.update({"w_up": f + "up", "b_up": f + "up.b", "w_down": f + "down", "b_down": f + "down.b"})
+    return n
+
+
+def _zovozen_sizes(ls, key: str) -> List[int]:
+    a, b = ls.branches
+    if key == "w_in":
+        return [a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim, a.heads * a.vdim, b.heads * b.dim, b.heads * b.dim,
+                b.heads * b.vdim, b.heads * b.vdim, b.heads, b.heads]
+    if key == "b_qkv":
+        return [a.heads * a.dim, a.kv_heads * a.dim, a.kv_heads * a.vdim]
+    return [b.heads, b.heads]
+
+
+def _load_zovozen_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) -> StageWeights:
+    w = StageWeights(spec, plan)
+    get = lambda name: rd.get(name).to(device=device, dtype=dtype)
+    w.embed, w.final_norm_w = get("embed"), get("final.norm")
+    w.lm_head = w.embed
+    for i in plan.layers:
+        ls, l = spec.layer_specs[i], {}
+        for k, names in _zovozen_layer_names(ls, f"l{i}.").items():
+            if isinstance(names, tuple):
+                l[k] = torch.cat([get(x) for x in names], dim=0)
+            elif isinstance(names, list):
+                l[k] = torch.stack([get(x) for x in names], dim=0)
+            else:
+                l[k] = get(names)
+        for k, sizes in (("w_in", _zovozen_sizes(ls, "w_in")), ("b_qkv", _zovozen_sizes(ls, "b_qkv"))):
+            if l[k].shape[0] != sum(sizes):
+                raise ValueError(f"layer {i}: the mixer's projections have {l[k].shape[0]} rows, the config says {sum(sizes)}")
+        if ls.moe is not None and l["w_router"].shape[0] != ls.moe.outputs:
+            raise ValueError(f"layer {i}: the router has {l['w_router'].shape[0]} outputs, the config says {ls.moe.outputs}")
+        w.layers.append(l)
+    return w
+
+
+def export_zovozen_state_dict(w: StageWeights) -> Dict[str, torch.Tensor]:
+    """Logical -> checkpoint names (tests, `save` of random models)."""
+    spec = w.spec
+    sd = {"embed": w.embed, "final.norm": w.final_norm_w}
+    for i, l in zip(w.plan.layers, w.layers):
+        ls = spec.layer_specs[i]
+        for k, names in _zovozen_layer_names(ls, f"l{i}.").items():
+            if isinstance(names, tuple):
+                for x, t in zip(names, torch.split(l[k], _zovozen_sizes(ls, k))):
+                    sd[x] = t
+            elif isinstance(names, list):
+                for x, t in zip(names, l[k]):
+                    sd[x] = t
+            else:
+                sd[names] = l[k]
+    return {k: v.detach().clone().contiguous() for k, v in sd.items()}
+
+
+def _random_zovozen_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
+    """Random weights with which every mechanism matters: projections at 1 / sqrt(fan-in), biases, norm weights, head
+    temperatures, mixing matrices, sinks and routing corrections of order one."""
+    H, V = spec.hidden_size, spec.vocab_size
+    w = StageWeights(spec, plan)
+    rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
+    one = lambda name, shape, std: torch.ones(shape, device=device, dtype=dtype) + rn(name, shape, std)
+    w.embed, w.final_norm_w = rn("embed", (V, H), 1.0), one("final.norm", (H,), 0.1)
+    w.lm_head = w.embed
+    for i in plan.layers:
+        ls, p = spec.layer_specs[i], f"layers.{i}."
+        a, b = ls.branches
+        sizes = _zovozen_sizes(ls, "w_in")
+        l: Dict[str, torch.Tensor] = {"ln1_w": one(p + "ln1_w", (H,), 0.2), "w_in": rn(p + "w_in", (sum(sizes), H), H ** -0.5)}
+        l["b_qkv"] = rn(p + "b_qkv", (sum(sizes[:3]),), 0.3)
+        l["q_norm_w"], l["k_norm_w"] = one(p + "q_norm_w", (sizes[0],), 0.2), one(p + "k_norm_w", (sizes[1],), 0.2)
+        l["talk"] = torch.eye(a.heads, device=device, dtype=dtype) + rn(p + "talk", (a.heads, a.heads), 0.3)
+        l["temp"], l["sink"] = one(p + "temp", (a.heads,), 0.3), rn(p + "sink", (a.heads,), 1.0)
+        l["w_o"], l["b_o"] = rn(p + "w_o", (H, a.heads * a.vdim), (a.heads * a.vdim) ** -0.5), rn(p + "b_o", (H,), 0.2)
+        l["b_if"] = rn(p + "b_if", (2 * b.heads,), 1.0)
+        l["o_norm_w"], l["w_o_r"] = one(p + "o_norm_w", (b.heads * b.vdim,), 0.1), rn(p + "w_o_r", (H, b.heads * b.vdim), (b.heads * b.vdim) ** -0.5)
+        if ls.has_ff:
+            l["ln2_w"] = one(p + "ln2_w", (H,), 0.2)
+        if ls.moe is not None:
+            e = ls.moe
+            l["w_router"], l["correction"] = rn(p + "w_router", (e.outputs, H), 2.0 * H ** -0.5), rn(p + "correction", (e.outputs,), 0.1)
+            l["w_gate_e"], l["w_up_e"] = rn(p + "w_gate_e", (e.experts, e.ff, H), 1.5 * H ** -0.5), rn(p + "w_up_e", (e.experts, e.ff, H), 1.5 * H ** -0.5)
+            l["w_down_e"] = rn(p + "w_down_e", (e.experts, H, e.ff), e.ff ** -0.5)
+            if e.shared_ff:
+                l["w_gate_s"], l["w_up_s"] = rn(p + "w_gate_s", (e.shared_ff, H), H ** -0.5), rn(p + "w_up_s", (e.shared_ff, H), H ** -0.5)
+                l["w_down_s"] = rn(p + "w_down_s", (H, e.shared_ff), e.shared_ff ** -0.5)
+        elif ls.ff:
+            l["w_up"], l["b_up"] = rn(p + "w_up", (ls.ff, H), H ** -0.5), rn(p + "b_up", (ls.ff,), 0.2)
+            l["w_down"], l["b_down"] = rn(p + "w_down", (H, ls.ff), ls.ff ** -0.5), rn(p + "b_down", (H,), 0.2)
+        w.layers.append(l)
+    return w
+
 
 def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, dtype) -> StageWeights:
     """Random weights of a hybrid stack, scaled so that activations stay of order one through any depth
@@ -348,6 +464,8 @@ def _random_hybrid_weights(spec: ModelSpec, plan: StagePlan, seed: int, device, 
         return _random_nufapel_weights(spec, plan, seed, device, dtype)
     if spec.family == "tezesun":
         return _random_tezesun_weights(spec, plan, seed, device, dtype)
+    if spec.family == "zovozen":
+        return _random_zovozen_weights(spec, plan, seed, device, dtype)
     H, V = spec.hidden_size, spec.vocab_size
     w = StageWeights(spec, plan)
     rn = lambda name, shape, std: _randn(name, shape, seed, device, dtype, std=std)
@@ -385,6 +503,8 @@ def _load_hybrid_weights(rd, spec: ModelSpec, plan: StagePlan, device, dtype) ->
         return _load_nufapel_weights(rd, spec, plan, device, dtype)
     if spec.family == "tezesun":
         return _load_tezesun_weights(rd, spec, plan, device, dtype)
+    if spec.family == "zovozen":
+        return _load_zovozen_weights(rd, spec, plan, device, dtype)
     w = StageWeights(spec, plan)
     get = lambda name: rd.get(name).to(device=device, dtype=dtype)
     if plan.has_embed or plan.has_head:

@@ -49,14 +49,16 @@ def rope(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, positions: torch
 
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, scale: float,
               window: int = 0, sink: bool = False, k_pos0: int = 0, temp=None, dist_bias=None, sink_logit=None,
-              keep_first: int = 0, softcap: float = 0.0) -> torch.Tensor:
+              keep_first: int = 0, softcap: float = 0.0, chunk: int = 0, head_mix=None) -> torch.Tensor:
     """One sequence. q [Tq, Hq, D] are the tokens at absolute positions q_pos0.., k [Tk, Hkv, D] and
     v [Tk, Hkv, Dv] hold positions k_pos0..k_pos0+Tk-1 (reaching at least the last query). Causal, GQA.
     `window` > 0: a query at i sees the keys j with 0 <= i - j < window. `sink`: the softmax's
     denominator has one more term, exp(0), that carries no value (`sink_logit` [Hq]: exp(sink_logit) instead).
     `temp` [Hq] multiplies a head's scaled scores; `dist_bias` [distances, Hq] is added to the scaled score of a
     key at distance i - j (after `temp`). `keep_first`: with a window, the keys at positions below it stay visible.
-    `softcap` > 0: scaled scores become cap tanh(score / cap). Returns [Tq, Hq, Dv] fp32."""
+    `softcap` > 0: scaled scores become cap tanh(score / cap). `head_mix` [Hq, Hq]: the heads' scores (scaled, after
+    `temp`) are mixed, s_h <- sum_g head_mix[h, g] s_g, before the mask. `chunk` > 0: a query sees only the keys of its own
+    chunk of that many positions (counted from position 0). Returns [Tq, Hq, Dv] fp32."""
     Tq, Hq, D = q.shape
     Tk, Hkv, _ = k.shape
     g = Hq // Hkv
@@ -71,7 +73,11 @@ def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, q_pos0: int, sc
         s = s * temp.float().view(Hq, 1, 1)
     if dist_bias is not None:
         s = s + dist_bias.float()[(qpos - kpos).clamp(min=0)].permute(2, 0, 1)
+    if head_mix is not None:
+        s = torch.einsum("hg,gqk->hqk", head_mix.float(), s)
     hidden = kpos > qpos
+    if chunk and chunk > 0:
+        hidden = hidden | (torch.div(qpos, chunk, rounding_mode="floor") != torch.div(kpos, chunk, rounding_mode="floor"))
     if window and window > 0:
         hidden = hidden | ((qpos - kpos >= window) & (kpos >= keep_first))
     s = s.masked_fill(hidden.unsqueeze(0), float("-inf"))
@@ -165,20 +171,26 @@ def matrix_memory(q, k, v, log_i, log_f, S, n, m):
     return out, S, n, m
 
 
-def moe_route(scores: torch.Tensor, top: int, groups: int, keep: int, scale: float):
-    """scores [T, E] fp32 (sigmoids of the router's logits) -> (experts [T, top] int64, weights [T, top] fp32). Experts
-    are split into `groups` contiguous blocks of equal size; a block is ranked by its best two scores added up; experts
-    outside the `keep` best blocks are out of the running; of the rest the `top` highest are taken, each weighted by
-    score / (sum of the taken scores + 1e-20) * scale. Equal scores go to the lower index."""
+def moe_route(scores: torch.Tensor, top: int, groups: int, keep: int, scale: float, correction=None, group_rank: int = 2,
+              renorm: bool = True):
+    """scores [T, E] fp32 (sigmoids or a softmax of the router's logits) -> (experts [T, top] int64, weights [T, top] fp32).
+    The choice goes by score + `correction` [E] (the score itself without one). Experts are split into `groups` contiguous
+    blocks of equal size; a block is ranked by its best `group_rank` choice scores added up; experts outside the `keep` best
+    blocks are out of the running (whatever their choice score's sign); of the rest the `top` highest are taken, each
+    weighted by its score: score / (sum of the taken scores + 1e-20) * scale, or score * scale with `renorm` off. Equal
+    choice scores go to the lower index."""
     T, E = scores.shape
     per = E // groups
     sf = scores.float()
-    gs = sf.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+    ch = sf if correction is None else sf + correction.float()
+    gs = ch.view(T, groups, per).topk(min(group_rank, per), dim=-1).values.sum(-1)
     order = torch.argsort(gs, dim=-1, descending=True, stable=True)[:, :keep]
     allowed = torch.zeros(T, groups, dtype=torch.bool, device=scores.device).scatter_(1, order, True)
-    masked = sf.masked_fill(~allowed.repeat_interleave(per, dim=1), -1.0)
+    masked = ch.masked_fill(~allowed.repeat_interleave(per, dim=1), float("-inf"))
     idx = torch.argsort(masked, dim=-1, descending=True, stable=True)[:, :top]
     val = sf.gather(1, idx)
+    if not renorm:
+        return idx, val * scale
     return idx, val / (val.sum(-1, keepdim=True) + 1e-20) * scale
 
 
