@@ -39,6 +39,19 @@ scaled by learned vectors and added together) run through `_layers_par`: per lay
              -> o GEMM;   up GEMM -> xIELU -> down GEMM (reads n itself)
              -> h += ls1 * mixer + ls2 * ff, the slot's carried n saved, and the next layer's n (one kernel)
 
+Stacks that norm their sublayers' OUTPUTS only (`spec.post_norm`: the sublayers read the stream itself) run through
+`_layers_post`: per layer
+
+    x (fp32, and in the GEMMs' type) -> ONE input GEMM (all projections of both mixers, biases in the epilogue)
+             -> [ q / k norms over the whole projection + rotation + unit values + the head mix folded into the query
+                  + cache write (one kernel) -> attention with chunked mask, learned sink and output gate -> o GEMM
+                  beside   matrix memory (exponential gates) -> per-head norm * weight * gate -> o GEMM ]
+             -> x += rms(a left + b right) w, and x in the GEMMs' type (one kernel)
+             -> [ up GEMM -> squared relu -> down GEMM
+                | router + shared gate / up GEMM -> route -> plan -> the experts' GEMMs over sorted rows -> weighted sum with
+                  the identity experts' share of x;  silu(gate) * up -> shared down GEMM ]
+             -> x += rms(ff) w
+
 Matrix products take bf16 operands (or fp32: `dtype="fp32"`, everything in true 32-bit) and accumulate in
 fp32; norms, scores, softmax, value mixing, gates, decays and states are fp32 in both modes.
 """
@@ -138,8 +151,23 @@ class HybridGpuStage(GpuStage):
             self._attn_of_run = [ls if ls.kind == "attention" else None for ls in self.specs]
         self.gated = spec.norm_kind == "dyt"
         self.par = spec.parallel_block
+        self.post = spec.post_norm
         self.runs = spec.layer_runs()
-        if self.par:
+        if self.post:
+            self.mfma_attn = [False] * len(self.specs)
+            self._attn_of_run = [ls.branches[0] for ls in self.specs]
+            # attention on the matrix cores in bf16 where a head's query row (all key heads side by side when the head mix is
+            # folded into it) is a multiple of 8; other sizes, and the fp32 mode, on the one-wave-per-(token, head) kernel.
+            # DLIA_POST_TILE_ATTN=0: all on that (A/B)
+            tile_ok = dtype == "bf16" and os.environ.get("DLIA_POST_TILE_ATTN", "1") != "0"
+            for i, a in zip(plan.layers, self._attn_of_run):
+                if self._query_row(a) > 1024:
+                    raise ValueError(f"layer {i}: a head's query row of {self._query_row(a)} entries (key heads x key size, with mixed heads) is beyond 1024")
+            self._tile = [tile_ok and self._query_row(a) % 8 == 0 and a.vdim <= 512 for a in self._attn_of_run]
+            self._load_post(weights, f32, mat)
+        if self.post:
+            pass
+        elif self.par:
             self.mfma_attn = [False] * len(self.specs)
             # attention layers whose sizes are multiples of 8 run on the matrix cores in bf16 (values key-contiguous in the
             # cache); other sizes, and the fp32 mode, on the one-wave-per-(token, head) kernel. DLIA_PAR_TILE_ATTN=0: all on that (A/B)
@@ -208,6 +236,11 @@ class HybridGpuStage(GpuStage):
             if ls.kind == "rglru":
                 st += (torch.zeros(max_slots + 1, max(ls.conv - 1, 1), ls.rec_width, device=dev), torch.zeros(max_slots + 1, ls.rec_width, device=dev))
             self.rec.append(st)
+        for ls in (self.specs if self.post else []):
+            # the matrix memory's state (its normaliser as one more column) and running maxima
+            b = ls.branches[1]
+            self.rec.append((torch.zeros(max_slots + 1, b.heads, b.dim, b.vdim + 1, device=dev),
+                             torch.zeros(max_slots + 1, b.heads, 128, device=dev)))
         for ls in ([spec.layer_specs[li] for li, _ in self.runs] if self.gated else []):
             if ls.kind == "general_delta":
                 self.rec.append((torch.zeros(max_slots + 1, ls.heads, ls.dim, ls.dim, device=dev),))
@@ -215,7 +248,7 @@ class HybridGpuStage(GpuStage):
                 b = ls.branches[1]
                 self.rec.append((torch.zeros(max_slots + 1, b.heads, b.dim, b.vdim + 1, device=dev),
                                  torch.zeros(max_slots + 1, b.heads, 128, device=dev)))
-        for ls in ([] if (self.gated or self.par) else self.specs):
+        for ls in ([] if (self.gated or self.par or self.post) else self.specs):
             if ls.kind == "delta":
                 C = 2 * ls.kv_heads * ls.dim + ls.heads * ls.vdim
                 self.rec.append((torch.zeros(max_slots + 1, max(ls.conv - 1, 1), C, device=dev),
@@ -270,6 +303,8 @@ class HybridGpuStage(GpuStage):
 
     # ---- workspaces ---------------------------------------------------------------------------------------
     def _new_work(self, rows: int):
+        if self.post:
+            return self._new_work_post(rows)
         if self.par:
             return self._new_work_par(rows)
         if self.gated:
@@ -309,7 +344,7 @@ class HybridGpuStage(GpuStage):
 
     def _decode_state_bytes(self) -> int:
         n = 0
-        if self.gated or self.par:
+        if self.gated or self.par or self.post:
             per_row = sum(t.numel() * t.element_size() for t in vars(self.wk0).values() if torch.is_tensor(t)) // self.max_tokens
             return sum(B * (per_row + 4 * self.vocab_pad) for B in self.graph_sizes)
         for B in self.graph_sizes:
@@ -321,6 +356,17 @@ class HybridGpuStage(GpuStage):
     def allocate_kv(self, num_blocks: int):
         dev, at = self.device, self.act_dtype
         self.num_blocks = int(num_blocks)
+        if self.post:
+            # keys: with the head mix folded into the query every head reads ALL key heads, so a token's keys are one row;
+            # values per key / value head, key-contiguous where the matrix-core kernel reads them
+            self.kv = []
+            for a, p, tile in zip(self._attn_of_run, self.layers, self._tile):
+                G, gk = a.kv_heads, 1 if p["mix"] is not None else a.kv_heads
+                kc = torch.zeros(self.num_blocks, gk, BLOCK, G * a.dim // gk, device=dev, dtype=at)
+                vc = torch.zeros(self.num_blocks, G, a.vdim, BLOCK, device=dev, dtype=at) if tile else \
+                    torch.zeros(self.num_blocks, G, BLOCK, a.vdim, device=dev, dtype=at)
+                self.kv.append((kc, vc))
+            return
         if self.par:
             # attention: key rows hold a head's score maps side by side, value rows apart; latent attention: ONE row per token,
             # the normed latent followed by the rotated key part (the values are the row's first entries)
@@ -370,6 +416,8 @@ class HybridGpuStage(GpuStage):
 
     def _layers(self, wk: _HybridWork, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int, splits: int,
                 alone: bool = False, lead_decode: int = 0):
+        if self.post:
+            return self._layers_post(wk, T, B, tok_pos, tok_seq, q_start, ctx, slots, max_q)
         if self.par:
             return self._layers_par(wk, T, B, tok_pos, tok_seq, q_start, ctx, slots, max_q)
         if self.gated:
@@ -826,6 +874,186 @@ class HybridGpuStage(GpuStage):
                 self.layer_outputs.append(h.clone())
         return None
 
+    # ---- stacks with norms on the sublayers' outputs only --------------------------------------------------------------
+    @staticmethod
+    def _query_row(a) -> int:
+        """Entries of one head's query as the attention kernel reads it: with mixed heads or head temperatures the mix is carried
+        by the query, which then holds a part for every key head."""
+        return a.kv_heads * a.dim if (a.head_mix or a.head_temp) else a.dim
+
+    def _load_post(self, weights: StageWeights, f32, mat):
+        """Device weights of a post-norm stack. Everything that reads the mixers' input is ONE matrix with the left branch's
+        q | k | v biases in its epilogue; the router and the shared expert's gate | up are one more. What scores, norms and the
+        recurrence need in fp32 (norm weights, the head mix, sinks, gate biases, rotation tables, routing corrections) stays
+        fp32 in both modes."""
+        from .rope import rope_table
+        spec, dev = self.spec, self.device
+        self.embed, self.pos_embed = mat(weights.embed), None
+        self.lm_head, self.lm_head_p = self.embed, None
+        self.final_norm_w = f32(weights.final_norm_w)
+        self.vocab_pad = packing.padded_n(spec.vocab_size)
+        self.layers = []
+        tables: Dict[tuple, tuple] = {}
+        for i, ls in enumerate(self.specs):
+            l = weights.layers[i]
+            a, b = ls.branches
+            p: Dict[str, object] = {"ln1_w": f32(l["ln1_w"])}
+            w_in = mat(l["w_in"])
+            b_in = torch.zeros(w_in.shape[0], device=dev)
+            if a.proj_bias:
+                b_in[:l["b_qkv"].numel()] = f32(l["b_qkv"])
+            self._matrix(p, "w_in", w_in, b_in)
+            self._matrix(p, "w_o", mat(l["w_o"]), f32(l["b_o"]) if a.proj_bias else None)
+            self._matrix(p, "w_o_r", mat(l["w_o_r"]), None)
+            p["q_norm_w"], p["k_norm_w"] = (f32(l["q_norm_w"]), f32(l["k_norm_w"])) if a.qk_norm else (None, None)
+            # score_h = sum_g talk[h, g] temp[g] scale (q_g . k): the mix, the temperatures and the scale are one matrix
+            p["mix"] = None
+            if a.head_mix or a.head_temp:
+                m = f32(l["talk"]) if a.head_mix else torch.eye(a.heads, device=dev)
+                if a.head_temp:
+                    m = m * f32(l["temp"]).view(1, -1)
+                p["mix"] = (m * a.scale).contiguous()
+            p["sink"] = (f32(l["sink"]) if a.sink_learned else torch.zeros(a.heads, device=dev)) if a.sink else None
+            if a.rope_dims:
+                key = (a.rope_dims, a.rope_base, a.rope_scaling)
+                if key not in tables:
+                    tables[key] = tuple(t.contiguous() for t in rope_table(a.rope_dims, a.rope_base, a.rope_scaling, self.max_seq_len, dev))
+                p["cos"], p["sin"] = tables[key]
+            else:
+                p["cos"] = p["sin"] = None
+            p["b_if"], p["o_norm_w"] = f32(l["b_if"]), f32(l["o_norm_w"])
+            if ls.has_ff:
+                p["ln2_w"] = f32(l["ln2_w"])
+            if ls.moe is not None:
+                e = ls.moe
+                if e.outputs > 256:
+                    raise ValueError("up to 256 router outputs are supported")
+                ff_in = [mat(l["w_router"])] + ([mat(l["w_gate_s"]), mat(l["w_up_s"])] if e.shared_ff else [])
+                self._matrix(p, "w_ff", torch.cat(ff_in), None)
+                p["correction"] = f32(l["correction"]) if e.correction else None
+                p["w_gate_e"], p["w_up_e"], p["w_down_e"] = (mat(l[k]) for k in ("w_gate_e", "w_up_e", "w_down_e"))
+                if e.shared_ff:
+                    self._matrix(p, "w_down_s", mat(l["w_down_s"]), None)
+            elif ls.ff:
+                self._matrix(p, "w_up", mat(l["w_up"]), f32(l["b_up"]))
+                self._matrix(p, "w_down", mat(l["w_down"]), f32(l["b_down"]))
+            self.layers.append(p)
+            weights.layers[i] = {}
+        if self._packed and spec.hidden_size % 128 == 0:
+            self.lm_head_p = packing.pack_weight(self.lm_head)
+            self._shapes.append((self.vocab_pad, spec.hidden_size, False))
+
+    def _new_work_post(self, rows: int):
+        s, dev, at = self.spec, self.device, self.act_dtype
+        z = lambda n, dt=torch.float32: torch.zeros(max(int(n), 1), device=dev, dtype=dt)
+        B, H = min(rows, self.max_batch), s.hidden_size
+        zc = qc = oc = mc = m2 = yc = z2 = ac = sc = 1
+        pairs = tiles = ef = 0
+        part = 1                  # partial results of the key splits of single-token steps (any number of rows up to B)
+        for ls, p, tile in zip(self.specs, self.layers, self._tile):
+            a, b = ls.branches
+            zc, qc = max(zc, self._cols(p, "w_in")), max(qc, a.heads * self._query_row(a))
+            mc, m2, oc = max(mc, a.heads * a.vdim), max(m2, b.heads * b.vdim), max(oc, b.heads * (b.vdim + 2))
+            yc = max(yc, self._cols(p, "w_o"), self._cols(p, "w_o_r"))
+            if tile:
+                part = max([part] + [int(self.K.tile_attention_part_floats(b_, a.heads, a.kv_heads, a.vdim, 1)) for b_ in range(1, B + 1)])
+            if ls.moe is not None:
+                e = ls.moe
+                z2 = max(z2, self._cols(p, "w_ff"))
+                # (rows of the experts' sorted copies: whole tiles of 32 rows, or of 128 for steps with many rows)
+                pairs, ef = max(pairs, rows * e.top), max(ef, e.ff)
+                tiles = max(tiles, (rows * e.top + 31) // 32 + e.experts, 4 * ((rows * e.top + 127) // 128 + e.experts))
+                if e.shared_ff:
+                    sc, yc = max(sc, e.shared_ff), max(yc, self._cols(p, "w_down_s"))
+            elif ls.ff:
+                z2, ac, yc = max(z2, self._cols(p, "w_up")), max(ac, ls.ff), max(yc, self._cols(p, "w_down"))
+        ws_floats = self._ws_floats
+        if self._packed and rows > self.decode_rows:
+            for m_ in {rows, min(rows, 512), min(rows, 1024)}:
+                if m_ > self.decode_rows:
+                    ws_floats = max([ws_floats] + [int(self.K.gemm_ws_floats(m_, n_, k_)) for n_, k_, _ in self._shapes])
+        i32 = torch.int32
+        return SimpleNamespace(
+            h=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc),
+            qf=z(rows * qc, at if any(self._tile) else torch.float32), qf32=z(rows * qc if not all(self._tile) else 1),
+            o=z(rows * oc), mixed=z(rows * mc, at), mixed2=z(rows * m2, at), ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2),
+            act=z(rows * ac, at), acts=z(rows * sc, at), sel=z(pairs, i32), wts=z(pairs), pair_row=z(pairs, i32), tiles=z(1 + tiles, i32),
+            row_tok=z(32 * tiles, i32), eact=z(32 * tiles * ef, at), ey=z(32 * tiles * H), part=z(part), ws=z(ws_floats + 4096),
+            head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
+
+    def _layers_post(self, wk, T: int, B: int, tok_pos, tok_seq, q_start, ctx, slots, max_q: int):
+        K, eps, H = self.K, self.spec.norm_eps, self.spec.hidden_size
+        h, xn = wk.h[:T], wk.xn[:T]
+        view = lambda buf, cols: buf[:T * cols].view(T, cols)
+        keep = self.keep_layer_outputs and not torch.cuda.is_current_stream_capturing()
+        if keep:
+            self.layer_outputs = []
+        table = self.block_table
+        K.post_norm_add(xn, h, None, None, 1.0, 0.0, None, eps)         # the stream in the GEMMs' input type
+        for li, (ls, p) in enumerate(zip(self.specs, self.layers)):
+            a, b = ls.branches
+            Hh, G, d, dv = a.heads, a.kv_heads, a.dim, a.vdim
+            qn, kn, vn, gn, bn, bv = Hh * d, G * d, G * dv, (Hh * dv if a.out_gate else 0), b.heads * b.dim, b.heads * b.vdim
+            # columns of the input projection: left q | k | v | g, right q | k | v | g | i | f
+            c_g = qn + kn + vn
+            c_q = c_g + Hh * dv
+            c_k, c_v, c_rg, c_i, c_f = c_q + bn, c_q + 2 * bn, c_q + 2 * bn + bv, c_q + 2 * bn + 2 * bv, c_q + 2 * bn + 2 * bv + b.heads
+            z = view(wk.z, self._cols(p, "w_in"))
+            self._mm(wk, z, xn, p, "w_in")
+            kc, vc = self.kv[li]
+            tile, kd = self._tile[li], self._query_row(a)
+            qf = view(wk.qf if tile else (wk.qf32 if wk.qf.dtype != torch.float32 else wk.qf), Hh * kd)
+            mixed, mixed2, o = view(wk.mixed, Hh * dv), view(wk.mixed2, bv), view(wk.o, b.heads * (b.vdim + 2))
+            K.mix_prep(z, Hh, G, d, dv, p["q_norm_w"], p["k_norm_w"], eps, a.rope_dims, p["cos"], p["sin"], a.v_norm, p["mix"], qf, kc, vc,
+                       tile, tok_pos, tok_seq, table)
+            gate = z[:, c_g:c_g + gn] if a.out_gate else None
+            scale = 1.0 if p["mix"] is not None else a.scale
+            if tile:
+                K.tile_attention(mixed, qf, kd, kc, vc, q_start, ctx, slots, table, max_q, Hh, kd, dv, 1, scale, a.window or 0, 0, 0.0,
+                                 0.0, 1.0, eps, gate, wk.part, a.chunk, p["sink"])
+            else:
+                K.multi_attention(mixed, qf, kd, kc, vc, 0, tok_pos, tok_seq, table, Hh, kd, dv, 1, scale, a.window or 0, 0, 0.0, 0.0,
+                                  1.0, eps, gate, a.chunk, p["sink"])
+            ya, yb = view(wk.ya, self._cols(p, "w_o")), view(wk.yb, self._cols(p, "w_o_r"))
+            self._mm(wk, ya, mixed, p, "w_o")
+            K.state_scan(1, o, z, None, self.rec[li][0], self.rec[li][1], p["b_if"], None, q_start, ctx, slots, b.heads, b.dim, b.vdim,
+                         c_q, c_k, c_v, 0, c_i, c_f, b.gate_cap, b.scale, max_q, self.wmode == "bf16")
+            K.headnorm_gate(mixed2, o, z[:, c_rg:c_rg + bv], p["o_norm_w"], b.heads, b.vdim, 2, eps)
+            self._mm(wk, yb, mixed2, p, "w_o_r")
+            sa, sb = ls.branch_scales or (1.0, 1.0)
+            K.post_norm_add(xn, h, ya[:, :H], yb[:, :H], sa, sb, p["ln1_w"], eps)
+            if ls.moe is not None:
+                e = ls.moe
+                z2 = view(wk.z2, self._cols(p, "w_ff"))
+                self._mm(wk, z2, xn, p, "w_ff")
+                # row tiles: 128 rows through the LDS-tiled kernel when the step has many rows (bf16, inner sizes in whole
+                # k-steps), else 32 rows through the register-tiled kernels; at most nt tiles hold a row
+                tr = 128 if (self.wmode == "bf16" and T * e.top >= 1024 and H % 32 == 0 and e.ff % 32 == 0) else 32
+                nt = (T * e.top + tr - 1) // tr + e.experts
+                eact, ey, ya = wk.eact[:tr * nt * e.ff].view(tr * nt, e.ff), wk.ey[:tr * nt * H].view(tr * nt, H), view(wk.ya, H)
+                K.moe_route(wk.sel, wk.wts, z2[:, :e.outputs], e.top, e.groups, e.keep, e.scale, p["correction"], e.score == "softmax",
+                            e.group_rank, e.renorm)
+                K.moe_plan(wk.tiles, wk.row_tok, wk.pair_row, wk.sel, T * e.top, e.top, e.experts, tr)
+                K.moe_up(eact, xn, p["w_gate_e"], p["w_up_e"], wk.tiles, wk.row_tok, nt, e.limit if e.act != "silu" else 0.0, tr)
+                K.moe_down(ey, eact, p["w_down_e"], wk.tiles, wk.row_tok, nt, tr)
+                K.moe_combine(ya, ey, wk.pair_row, wk.wts, e.top, h if e.identity else None)
+                yb = None
+                if e.shared_ff:
+                    acts, yb = view(wk.acts, e.shared_ff), view(wk.yb, self._cols(p, "w_down_s"))
+                    K.unary_act(acts, z2[:, e.outputs:e.outputs + 2 * e.shared_ff], 3)
+                    self._mm(wk, yb, acts, p, "w_down_s")
+                    yb = yb[:, :H]
+                K.post_norm_add(xn, h, ya, yb, 1.0, 1.0, p["ln2_w"], eps)
+            elif ls.ff:
+                z2, act, ya = view(wk.z2, self._cols(p, "w_up")), view(wk.act, ls.ff), view(wk.ya, self._cols(p, "w_down"))
+                self._mm(wk, z2, xn, p, "w_up")
+                K.unary_act(act, z2[:, :ls.ff], 2)
+                self._mm(wk, ya, act, p, "w_down")
+                K.post_norm_add(xn, h, ya[:, :H], None, 1.0, 0.0, p["ln2_w"], eps)
+            if keep:
+                self.layer_outputs.append(h.clone())
+        return None
+
     def _fold(self, wk, T: int, pend):
         return None
 
@@ -835,7 +1063,7 @@ class HybridGpuStage(GpuStage):
         if self.gated:
             K.dyt_gate(hx, wk.h[:T], None, None, None, None, None, None, None, self.final_norm_w, self.final_norm_b, rows_idx[:R],
                        self.final_norm_a, self.spec.norm_eps)
-        elif self.par:
+        elif self.par or self.post:
             K.norm32(hx, wk.h[:T], None, None, self.final_norm_w, rows_idx[:R], self.spec.norm_eps, 0.0)
         else:
             K.norm32(hx, wk.h[:T], None, None, self.final_norm_w, rows_idx[:R], self.spec.norm_eps, 1.0)

@@ -115,7 +115,8 @@ void headnorm_gate(Tensor out, const Tensor& o, const Tensor& gate, const Tensor
 void unary_act(Tensor act, const Tensor& z, int64_t kind) {
   DLIA_ON_DEVICE_OF(act);
   check_act(act, "act"); check_mat(act, "act"); check_fmat(z, "z");
-  DLIA_CHECK(z.size(0) >= act.size(0) && z.size(1) == act.size(1) && (kind == 0 || kind == 1), "unary_act: z [M, F], act [M, F], kind 0 or 1");
+  DLIA_CHECK(kind >= 0 && kind <= 3 && z.size(0) >= act.size(0) && z.size(1) == (kind == 3 ? 2 : 1) * act.size(1),
+             "unary_act: act [M, F] from z [M, F] (kinds 0 to 2) or from gate | up in z [M, 2 F] (kind 3)");
   dlia_unary_act(act.data_ptr(), is_f32(act), z.data_ptr<float>(), (int)act.size(0), (int)act.size(1), z.stride(0), act.stride(0), (int)kind,
                  cur_stream());
 }
@@ -202,15 +203,17 @@ void state_scan(int64_t rule, Tensor o, const Tensor& z, OptTensor wz, Tensor st
   DLIA_CHECK(rc == 0, "state_scan: key size ", d, " / value size ", dv, " beyond what the kernel splits (1024 rows, 128 column blocks)");
 }
 
-void moe_route(Tensor sel, Tensor wts, const Tensor& logits, int64_t top, int64_t groups, int64_t keep, double scale) {
+void moe_route(Tensor sel, Tensor wts, const Tensor& logits, int64_t top, int64_t groups, int64_t keep, double scale, OptTensor correction,
+               bool softmax, int64_t group_rank, bool renorm) {
   DLIA_ON_DEVICE_OF(sel);
   check_i32(sel, "sel"); check_f32(wts, "wts"); check_fmat(logits, "logits");
   const int64_t T = logits.size(0), E = logits.size(1);
   DLIA_CHECK(E >= 1 && E <= 256 && groups >= 1 && E % groups == 0 && keep >= 1 && keep <= groups && top >= 1 && top <= keep * (E / groups),
              "moe_route: up to 256 experts in equal groups, top within the kept groups");
-  DLIA_CHECK(sel.numel() >= T * top && wts.numel() >= T * top, "moe_route: sel / wts [T, top]");
+  DLIA_CHECK(sel.numel() >= T * top && wts.numel() >= T * top && (group_rank == 1 || group_rank == 2), "moe_route: sel / wts [T, top], groups ranked by 1 or 2 members");
   dlia_moe_route(sel.data_ptr<int>(), wts.data_ptr<float>(), logits.data_ptr<float>(), logits.stride(0), (int)T, (int)E, (int)top,
-                 (int)groups, (int)keep, (float)scale, cur_stream());
+                 (int)groups, (int)keep, (float)scale, opt_f32(correction, E, "correction"), softmax ? 1 : 0, (int)group_rank, renorm ? 1 : 0,
+                 cur_stream());
 }
 
 void moe_plan(Tensor tiles, Tensor row_tok, Tensor pair_row, const Tensor& sel, int64_t pairs, int64_t top, int64_t E, int64_t tile_rows) {
@@ -257,13 +260,19 @@ void moe_down(Tensor y, const Tensor& act, const Tensor& wd, const Tensor& tiles
                 (int)max_tiles, max_tiles > 64 ? 1 : 0, (int)wd.size(1), (int)wd.size(2), act.stride(0), (int)tile_rows, cur_stream());
 }
 
-void moe_combine(Tensor out, const Tensor& y, const Tensor& pair_row, const Tensor& wts, int64_t top) {
+void moe_combine(Tensor out, const Tensor& y, const Tensor& pair_row, const Tensor& wts, int64_t top, OptTensor x) {
   DLIA_ON_DEVICE_OF(out);
   check_fmat(out, "out"); check_f32(y, "y"); check_i32(pair_row, "pair_row"); check_f32(wts, "wts");
   const int64_t T = out.size(0), H = out.size(1);
   DLIA_CHECK(y.dim() == 2 && y.size(1) == H && pair_row.numel() >= T * top && wts.numel() >= T * top, "moe_combine: shapes");
+  const float* xp = nullptr; long ldx = 0;
+  if (x.has_value()) {      // what a choice without a row (an identity expert) returns
+    check_fmat(*x, "x");
+    DLIA_CHECK(x->size(0) >= T && x->size(1) == H, "moe_combine: x [T, H]");
+    xp = x->data_ptr<float>(); ldx = x->stride(0);
+  }
   dlia_moe_combine(out.data_ptr<float>(), y.data_ptr<float>(), pair_row.data_ptr<int>(), wts.data_ptr<float>(), (int)T, (int)H, (int)top,
-                   out.stride(0), cur_stream());
+                   out.stride(0), xp, ldx, cur_stream());
 }
 
 }  // namespace
@@ -277,11 +286,11 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("biased_attention(Tensor(a!) out, Tensor qkv, Tensor kcache, Tensor vcache, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int G, int d, int dv, float scale, Tensor? temp, Tensor? bias, Tensor? sink, Tensor? gate) -> ()");
   m.def("state_scan_blocks(int d, int ncols) -> int");
   m.def("state_scan(int rule, Tensor(a!) o, Tensor z, Tensor? wz, Tensor(b!) state, Tensor(c!)? mstate, Tensor b0, Tensor? b1, Tensor q_start, Tensor ctx, Tensor slots, int H, int d, int dv, int col_q, int col_k, int col_v, int col_a, int col_i, int col_f, float cap, float qscale, int max_q, bool quick) -> ()");
-  m.def("moe_route(Tensor(a!) sel, Tensor(b!) wts, Tensor logits, int top, int groups, int keep, float scale) -> ()");
+  m.def("moe_route(Tensor(a!) sel, Tensor(b!) wts, Tensor logits, int top, int groups, int keep, float scale, Tensor? correction=None, bool softmax=False, int group_rank=2, bool renorm=True) -> ()");
   m.def("moe_plan(Tensor(a!) tiles, Tensor(b!) row_tok, Tensor(c!) pair_row, Tensor sel, int pairs, int top, int E, int tile_rows) -> ()");
   m.def("moe_up(Tensor(a!) act, Tensor x, Tensor wg, Tensor wu, Tensor tiles, Tensor row_tok, int max_tiles, float limit, int tile_rows) -> ()");
   m.def("moe_down(Tensor(a!) y, Tensor act, Tensor wd, Tensor tiles, Tensor row_tok, int max_tiles, int tile_rows) -> ()");
-  m.def("moe_combine(Tensor(a!) out, Tensor y, Tensor pair_row, Tensor wts, int top) -> ()");
+  m.def("moe_combine(Tensor(a!) out, Tensor y, Tensor pair_row, Tensor wts, int top, Tensor? x=None) -> ()");
 }
 
 TORCH_LIBRARY_IMPL(dlia, CUDA, m) {

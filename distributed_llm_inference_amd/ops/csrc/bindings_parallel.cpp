@@ -148,15 +148,17 @@ void rope_cache_write(Tensor q, int64_t q_vecs, int64_t q_stride, int64_t q_off,
 void multi_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& kcache, const Tensor& vcache, int64_t v_off,
                      const Tensor& tok_pos, const Tensor& tok_seq, const Tensor& block_table, int64_t H, int64_t d, int64_t dv,
                      int64_t maps, double scale, int64_t window, int64_t keep_first, double softcap, double lam, double post, double eps,
-                     OptTensor gate) {
+                     OptTensor gate, int64_t chunk, OptTensor sink) {
   DLIA_ON_DEVICE_OF(out);
   check_act(out, "out"); check_mat(out, "out"); check_fmat(q, "q"); check_act(kcache, "kcache"); check_act(vcache, "vcache");
   check_i32(tok_pos, "tok_pos"); check_i32(tok_seq, "tok_seq"); check_i32(block_table, "block_table");
   const int64_t T = out.size(0);
   DLIA_CHECK(kcache.dim() == 4 && vcache.dim() == 4 && kcache.is_contiguous() && vcache.is_contiguous() && kcache.size(2) == 32 &&
-             vcache.size(2) == 32 && kcache.size(0) == vcache.size(0) && kcache.size(1) == vcache.size(1) &&
+             vcache.size(2) == 32 && kcache.size(0) == vcache.size(0) &&
              kcache.scalar_type() == vcache.scalar_type() && out.scalar_type() == kcache.scalar_type(), "multi_attention: caches [blocks, G, 32, row], output in their type");
-  const int64_t G = kcache.size(1), k_row = kcache.size(3), v_row = vcache.size(3);
+  // (the key cache may hold fewer heads than the value cache: one row of all key heads for queries that carry a mix of heads)
+  const int64_t G = vcache.size(1), Gk = kcache.size(1), k_row = kcache.size(3), v_row = vcache.size(3);
+  DLIA_CHECK(Gk >= 1 && H % Gk == 0 && chunk >= 0 && (chunk == 0 || keep_first == 0), "multi_attention: key heads divide the heads; a chunked mask keeps no first tokens");
   DLIA_CHECK((maps == 1 || maps == 2) && d >= 1 && maps * d <= 1024 && maps * d <= k_row && dv >= 1 && dv <= 512 && v_off >= 0 &&
              v_off + dv <= v_row, "multi_attention: 1 or 2 maps, maps * d <= 1024 inside the key row, dv <= 512 inside the value row");
   DLIA_CHECK(H >= 1 && G >= 1 && H % G == 0 && out.size(1) == H * dv && q.size(0) >= T && q_head >= maps * d &&
@@ -172,7 +174,7 @@ void multi_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& 
                        vcache.data_ptr(), (int)v_row, (int)v_off, is_f32(kcache), tok_pos.data_ptr<int>(), tok_seq.data_ptr<int>(),
                        block_table.data_ptr<int>(), (int)T, (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0),
                        (int)H, (int)G, (int)d, (int)dv, (int)maps, (float)scale, (int)window, (int)keep_first, (float)softcap,
-                       (float)lam, (float)post, (float)eps, gp, ldg, cur_stream());
+                       (float)lam, (float)post, (float)eps, gp, ldg, (int)Gk, (int)chunk, opt_f32(sink, H, "sink"), cur_stream());
 }
 
 // The same attention on the matrix cores: bf16, q [T, .] bf16, values key-contiguous in vt [blocks, G, dv, 32]; per sequence
@@ -180,7 +182,7 @@ void multi_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& 
 void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& kcache, const Tensor& vt, const Tensor& q_start,
                     const Tensor& ctx, const Tensor& slots, const Tensor& block_table, int64_t max_q, int64_t H, int64_t d, int64_t dv,
                     int64_t maps, double scale, int64_t window, int64_t keep_first, double softcap, double lam, double post, double eps,
-                    OptTensor gate, const std::optional<Tensor>& part) {
+                    OptTensor gate, const std::optional<Tensor>& part, int64_t chunk, OptTensor sink) {
   DLIA_ON_DEVICE_OF(out);
   check_mat(out, "out"); check_mat(q, "q");
   check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots"); check_i32(block_table, "block_table");
@@ -189,8 +191,10 @@ void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& k
              "tile_attention: bfloat16 on the GPU");
   const int64_t T = out.size(0), B = ctx.numel();
   DLIA_CHECK(kcache.dim() == 4 && vt.dim() == 4 && kcache.is_contiguous() && vt.is_contiguous() && kcache.size(2) == 32 && vt.size(3) == 32 &&
-             kcache.size(0) == vt.size(0) && kcache.size(1) == vt.size(1) && vt.size(2) == dv, "tile_attention: kcache [blocks, G, 32, row], vt [blocks, G, dv, 32]");
-  const int64_t G = kcache.size(1), k_row = kcache.size(3);
+             kcache.size(0) == vt.size(0) && (kcache.size(1) == vt.size(1) || kcache.size(1) == 1) && vt.size(2) == dv,
+             "tile_attention: kcache [blocks, G or 1, 32, row], vt [blocks, G, dv, 32]");
+  const int64_t G = vt.size(1), Gk = kcache.size(1), k_row = kcache.size(3);
+  DLIA_CHECK(chunk >= 0 && (chunk == 0 || keep_first == 0), "tile_attention: a chunked mask keeps no first tokens");
   DLIA_CHECK((maps == 1 || maps == 2) && d >= 8 && maps * d <= k_row && H >= 1 && H % G == 0 && out.size(1) == H * dv && q.size(0) >= T &&
              q_head >= maps * d && (H - 1) * q_head + maps * d <= q.size(1), "tile_attention: head geometry");
   DLIA_CHECK(q_start.numel() >= B + 1 && slots.numel() >= B && block_table.dim() == 2 && max_q >= 0 && max_q <= T && window >= 0 && keep_first >= 0,
@@ -208,7 +212,7 @@ void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& k
                                      vt.data_ptr(), q_start.data_ptr<int>(), ctx.data_ptr<int>(), slots.data_ptr<int>(), block_table.data_ptr<int>(),
                                      (int)B, (int)max_q, (int)block_table.size(1), (int)kcache.size(0), (int)block_table.size(0), (int)H, (int)G,
                                      (int)d, (int)dv, (int)maps, (float)scale, (int)window, (int)keep_first, (float)softcap, (float)lam,
-                                     (float)post, (float)eps, gp, ldg, pp, pn, cur_stream());
+                                     (float)post, (float)eps, gp, ldg, pp, pn, (int)Gk, (int)chunk, opt_f32(sink, H, "sink"), cur_stream());
   DLIA_CHECK(rc != 2, "tile_attention: a single-token step needs the workspace for its key splits (tile_attention_part_floats)");
   DLIA_CHECK(rc == 0, "tile_attention: sizes must be multiples of 8 (d, key row, q head stride, q row), maps * d <= 1024, dv <= 512");
 }
@@ -271,8 +275,8 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("par_norm(Tensor(a!)? out, Tensor(b!) out32, Tensor(c!) x, Tensor? ya, Tensor? yb, Tensor? ls1, Tensor? ls2, Tensor? w, Tensor(d!)? carry, Tensor tok_seq, float eps) -> ()");
   m.def("token_shift(Tensor(a!) out, Tensor n32, Tensor carry, Tensor mu, Tensor tok_pos, Tensor tok_seq) -> ()");
   m.def("rope_cache_write(Tensor(a!) q, int q_vecs, int q_stride, int q_off, Tensor(b!)? q_out, int q_cols, Tensor(c!) kv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols, bool v_t, Tensor(d!) kcache, Tensor(e!)? vcache, int dims, bool interleaved, Tensor? cos_t, Tensor? sin_t, Tensor tok_pos, Tensor tok_seq, Tensor block_table) -> ()");
-  m.def("multi_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vcache, int v_off, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate) -> ()");
-  m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, Tensor(b!)? part) -> ()");
+  m.def("multi_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vcache, int v_off, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, int chunk=0, Tensor? sink=None) -> ()");
+  m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, Tensor(b!)? part, int chunk=0, Tensor? sink=None) -> ()");
   m.def("tile_attention_part_floats(int B, int H, int G, int dv, int maps) -> int");
   m.def("rglru_scan(Tensor(a!) out, Tensor u, Tensor gates, Tensor ypre, Tensor clam, Tensor(b!) state, Tensor q_start, Tensor ctx, Tensor slots, int bw, int max_q, Tensor(c!)? ws) -> ()");
   m.def("rglru_scan_ws_floats(int rows, int B, int W) -> int");

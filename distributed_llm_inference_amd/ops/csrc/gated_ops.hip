@@ -90,7 +90,13 @@ __global__ __launch_bounds__(256) void unary_act_kernel(OT* __restrict__ act, co
   if (i >= n) return;
   const long m = i / F; const int c = (int)(i % F);
   const float x = z[m * ldz + c];
-  act[m * lda + c] = (OT)(kind == 0 ? 0.5f * x * (1.f + erff(x * 0.7071067811865476f)) : tanhf(x));
+  // 0: exact GELU, 1: tanh, 2: the square of relu, 3: silu(x) times the entry F columns further (gate | up side by side)
+  float y;
+  if (kind == 0) y = 0.5f * x * (1.f + erff(x * 0.7071067811865476f));
+  else if (kind == 1) y = tanhf(x);
+  else if (kind == 2) { const float r = fmaxf(x, 0.f); y = r * r; }
+  else y = x / (1.f + expf(-x)) * z[m * ldz + c + F];
+  act[m * lda + c] = (OT)y;
 }
 
 __global__ __launch_bounds__(256) void softcap_kernel(float* __restrict__ z, long n, int V, long ld, float cap) {

@@ -168,7 +168,7 @@ int dlia_state_scan(int rule, float* o, long ldo, const float* z, long ldz, cons
 
 // ---- moe.hip --------------------------------------------------------------------------------
 void dlia_moe_route(int* sel, float* wts, const float* logits, long ld, int T, int E, int top, int groups, int keep, float scale,
-                    hipStream_t stream);
+                    const float* corr, int softmax, int group_rank, int renorm, hipStream_t stream);
 void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows, int tile_rows,
                    hipStream_t stream);
 // tile_rows: 32 (register-tiled expert kernels, any type and shape) or 128 (LDS-tiled, bf16, K a multiple of 32, aligned rows)
@@ -178,7 +178,8 @@ void dlia_moe_down(float* y, const void* act, const void* wd, int f32, const int
                    int H, int F, long lda, int tile_rows, hipStream_t stream);
 // (wide: 128 / 256 output columns per workgroup, for steps with many rows; else 64)
 void dlia_moe_combine(float* out, const float* y, const int* pair_row, const float* wts, int T, int H, int top, long ldo,
-                      hipStream_t stream);
+                      const float* x, long ldx, hipStream_t stream);
+
 
 
 // ---- parallel_ops.hip (parallel layers on one norm, token shift, rotation + cache write, attention over score maps, RG-LRU) ----
@@ -196,13 +197,13 @@ void dlia_multi_attention(void* out, long ldo, const float* q, long ldq, int q_h
                           const void* vcache, int v_row, int v_off, int f32, const int* tok_pos, const int* tok_seq,
                           const int* block_table, int T, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
                           int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
-                          const float* gate, long ldg, hipStream_t stream);
+                          const float* gate, long ldg, int Gk, int chunk, const float* sink, hipStream_t stream);
 // bf16 on the matrix cores; values key-contiguous in `vt` [blocks, G, dv, 32]. Returns 1 (nothing launched) for sizes it does not take.
 int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head, const void* kcache, int k_row, const void* vt,
                         const int* q_start, const int* ctx, const int* slots, const int* block_table, int B, int max_q,
                         int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv, int maps, float scale,
                         int window, int keep_first, float softcap, float lam, float post, float eps, const float* gate, long ldg,
-                        float* part, long part_floats, hipStream_t stream);
+                        float* part, long part_floats, int Gk, int chunk, const float* sink, hipStream_t stream);
 // key splits of a single-token step of B rows (the workspace `part` holds B * H * maps * splits * (dv + 2) floats)
 int dlia_tile_attention_splits(int B, int H, int G);
 void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg, const float* ypre,
@@ -211,6 +212,14 @@ void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu,
 long dlia_rglru_scan_ws_floats(int rows, int B, int W);
 void dlia_xielu(void* act, int out_f32, const float* z, int M, int F, long ldz, long lda, const float* pq, hipStream_t stream);
 void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStream_t stream);
+// ---- postnorm_ops.hip (norms on the sublayers' outputs only; q / k / v preparation of an attention mixer) ----
+void dlia_post_norm_add(void* out, int out_f32, long ldo, float* x, long ldx, const float* ya, long ldya, const float* yb, long ldyb,
+                        float a, float b, const float* w, int T, int H, float eps, hipStream_t stream);
+// Returns 1 (nothing launched) when a token's q and k do not fit a workgroup's LDS.
+int dlia_mix_prep(const float* z, long ldz, int T, int H, int G, int d, int dv, const float* qw, const float* kw, float eps, int dims,
+                  const float* cos_t, const float* sin_t, int table_pos, int v_unit, const float* mix, void* q_out, int q_f32, long ldqo,
+                  void* kcache, int Gk, void* vcache, int v_t, int cache_f32, const int* tok_pos, const int* tok_seq,
+                  const int* block_table, int max_blocks, int num_blocks, int table_rows, hipStream_t stream);
 // ---- misc.hip -------------------------------------------------------------------------
 void dlia_advance_i32(int* x, int n, int delta, hipStream_t stream);
 void dlia_scatter_rows_i32(int* dst, const int* rows, const int* src, int nrows, int ncols, int dst_rows, hipStream_t stream);

@@ -1,17 +1,22 @@
 // Routed feed-forward (mixture of experts) without a host round trip: routing, a plan that sorts the step's (token, choice)
 // pairs by expert into 32-row tiles, the experts' two GEMMs over those tiles, and the weighted sum per token.
 //
-//   moe_route    one thread per token. Scores are sigmoids of the fp32 router logits. Experts are split into `groups` contiguous blocks of
-//                equal size; a block is ranked by its best two scores added up; the `keep` best blocks stay; the `top`
-//                best experts of those are chosen (equal scores: the lower index), weighted score / (sum + 1e-20) * scale.
-//   moe_plan     one workgroup. Counts the pairs per expert, lays the experts' row ranges out one after the other, each
+//   moe_route    one thread per token. Scores are sigmoids of the fp32 router logits, or their softmax over all router outputs.
+//                The choice goes by score + correction[e] when a correction is given. Experts are split into `groups`
+//                contiguous blocks of equal size; a block is ranked by its best `group_rank` (1 or 2) choice scores added up;
+//                the `keep` best blocks stay; the `top` best experts of those are chosen (equal scores: the lower index),
+//                weighted score / (sum + 1e-20) * scale, or score * scale without the division.
+//   moe_plan     one workgroup. Pairs whose choice is not a real expert (an identity expert: index >= E) get row -1 and no
+//                place in a tile. Counts the pairs per expert, lays the experts' row ranges out one after the other, each
 //                padded to whole 32-row tiles, and writes for every padded row its token (or -1), for every pair its row,
 //                for every tile its expert; tiles[0] holds the number of tiles. Rows of one expert are in no fixed order:
 //                every row is computed on its own, so the order does not reach the results.
 //   moe_up       grid (column blocks, tiles): act[row, f] = g s(1.702 g) (u + 1), g = min(x . Wg[e][f], limit),
-//                u = clamp(x . Wu[e][f], -limit, limit), x the row's token; gate and up accumulate over the same A fragments.
+//                u = clamp(x . Wu[e][f], -limit, limit), x the row's token; with limit <= 0 the plain silu(g) * u.
+//                Gate and up accumulate over the same A fragments.
 //   moe_down     y[row, c] = act[row] . Wd[e][c] in fp32.
-//   moe_combine  out[t, :] = sum over the token's choices of weight * y[row, :], in the order of the choices (fp32).
+//   moe_combine  out[t, :] = sum over the token's choices of weight * y[row, :], in the order of the choices (fp32); a choice
+//                without a row (an identity expert) contributes weight * x[t, :].
 // Operands are bf16 (16x16x32 MFMA) or fp32 (16x16x4 MFMA, true 32-bit), fragments read straight from the K-contiguous rows.
 #include "common.h"
 #include "frag.h"
@@ -23,46 +28,67 @@ constexpr int kMoeMaxExperts = 256;
 constexpr int kMoeRows = 32;           // rows of a plan tile (steps with few rows), kMoeBigRows for the LDS-tiled kernel
 constexpr int kMoeBigRows = 128;
 
+// An expert's activation from its gate and up pre-activations.
+__device__ __forceinline__ float expert_act(float g, float u, float limit) {
+  if (limit > 0.f) {
+    const float gv = fminf(g, limit), uv = fminf(fmaxf(u, -limit), limit);
+    return gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f);
+  }
+  return g / (1.f + expf(-g)) * u;
+}
+
 __global__ __launch_bounds__(64) void moe_route_kernel(int* __restrict__ sel, float* __restrict__ wts,
                                                        const float* __restrict__ logits, long ld, int T, int E, int top,
-                                                       int groups, int keep, float scale) {
+                                                       int groups, int keep, float scale, const float* __restrict__ corr,
+                                                       int softmax, int group_rank, int renorm) {
   const int t = blockIdx.x * 64 + threadIdx.x;
   if (t >= T) return;
   const float* z = logits + (long)t * ld;
   const int per = E / groups;
-  auto score = [&](int e) { return 1.f / (1.f + expf(-z[e])); };
+  float zmax = 0.f, zinv = 1.f;
+  if (softmax) {
+    zmax = -INFINITY;
+    for (int e = 0; e < E; ++e) zmax = fmaxf(zmax, z[e]);
+    float sum = 0.f;
+    for (int e = 0; e < E; ++e) sum += expf(z[e] - zmax);
+    zinv = 1.f / sum;
+  }
+  auto score = [&](int e) { return softmax ? expf(z[e] - zmax) * zinv : 1.f / (1.f + expf(-z[e])); };
+  auto choice = [&](int e) { return corr ? score(e) + corr[e] : score(e); };
   // the groups that stay: `keep` times the best group not yet taken
   unsigned long long gmask[4] = {0ull, 0ull, 0ull, 0ull};
   for (int r = 0; r < keep; ++r) {
-    int best = -1; float bs = -1.f;
+    int best = -1; float bs = -INFINITY;
     for (int g = 0; g < groups; ++g) {
       if (gmask[g >> 6] >> (g & 63) & 1ull) continue;
-      float a = -1.f, b = -1.f;                       // the block's best two scores
+      float a = -INFINITY, b = -INFINITY;             // the block's best two choice scores
       for (int e = g * per; e < (g + 1) * per; ++e) {
-        const float s = score(e);
+        const float s = choice(e);
         if (s > a) { b = a; a = s; } else if (s > b) b = s;
       }
-      const float gs = a + (b > 0.f ? b : 0.f);
-      if (gs > bs) { bs = gs; best = g; }
+      const float gs = a + (group_rank >= 2 && b > -INFINITY ? b : 0.f);
+      if (best < 0 || gs > bs) { bs = gs; best = g; }
     }
     if (best >= 0) gmask[best >> 6] |= 1ull << (best & 63);
   }
   unsigned long long emask[4] = {0ull, 0ull, 0ull, 0ull};
   float total = 0.f;
   for (int r = 0; r < top; ++r) {
-    int best = 0; float bs = -1.f;
+    int best = -1; float bs = -INFINITY;
     for (int e = 0; e < E; ++e) {
       const int g = e / per;
       if (!(gmask[g >> 6] >> (g & 63) & 1ull) || (emask[e >> 6] >> (e & 63) & 1ull)) continue;
-      const float s = score(e);
-      if (s > bs) { bs = s; best = e; }
+      const float s = choice(e);
+      if (best < 0 || s > bs) { bs = s; best = e; }
     }
+    if (best < 0) best = 0;
     emask[best >> 6] |= 1ull << (best & 63);
+    const float w = score(best);
     sel[(long)t * top + r] = best;
-    wts[(long)t * top + r] = bs;
-    total += bs;
+    wts[(long)t * top + r] = w;
+    total += w;
   }
-  const float inv = scale / (total + 1e-20f);
+  const float inv = renorm ? scale / (total + 1e-20f) : scale;
   for (int r = 0; r < top; ++r) wts[(long)t * top + r] *= inv;
 }
 
@@ -74,7 +100,8 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ tiles,
   __shared__ int ntiles;
   for (int e = threadIdx.x; e < E; e += 1024) { count[e] = 0; fill[e] = 0; }
   __syncthreads();
-  for (int i = threadIdx.x; i < pairs; i += 1024) atomicAdd(&count[sel[i]], 1);
+  for (int i = threadIdx.x; i < pairs; i += 1024)
+    if (sel[i] < E) atomicAdd(&count[sel[i]], 1);
   __syncthreads();
   if (threadIdx.x == 0) {
     int at = 0, nt = 0;
@@ -93,6 +120,7 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(int* __restrict__ tiles,
   __syncthreads();
   for (int i = threadIdx.x; i < pairs; i += 1024) {
     const int e = sel[i];
+    if (e >= E) { pair_row[i] = -1; continue; }                      // (an identity expert: no row)
     const int r = start[e] + atomicAdd(&fill[e], 1);
     if (r < max_rows && r < used) { row_tok[r] = i / top; pair_row[i] = r; }
   }
@@ -164,8 +192,7 @@ __global__ __launch_bounds__(256) void moe_up_kernel(OT* __restrict__ act, const
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const int row = tile * kMoeTile + i * 16 + kq * 4 + r;
-        const float gv = fminf(ag[i][j][r], limit), uv = fminf(fmaxf(au[i][j][r], -limit), limit);
-        act[(long)row * lda + col] = (OT)(gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f));
+        act[(long)row * lda + col] = (OT)expert_act(ag[i][j][r], au[i][j][r], limit);
       }
     }
 }
@@ -309,8 +336,7 @@ __global__ __launch_bounds__(256) void moe_big_kernel(bf16* __restrict__ act_out
         for (int j = 0; j < 4; ++j) {
           const int col = n0 + j * 16 + r16;
           if (col >= N) continue;
-          const float gv = fminf(acc[i][j][r], limit), uv = fminf(fmaxf(acc[i][j + 4][r], -limit), limit);
-          act_out[row * ldo + col] = (bf16)(gv / (1.f + expf(-1.702f * gv)) * (uv + 1.f));
+          act_out[row * ldo + col] = (bf16)expert_act(acc[i][j][r], acc[i][j + 4][r], limit);
         }
       } else {
 #pragma unroll
@@ -324,11 +350,14 @@ __global__ __launch_bounds__(256) void moe_big_kernel(bf16* __restrict__ act_out
 
 __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ out, const float* __restrict__ y,
                                                           const int* __restrict__ pair_row, const float* __restrict__ wts,
-                                                          int H, int top, long ldo) {
+                                                          int H, int top, long ldo, const float* __restrict__ x, long ldx) {
   const int t = blockIdx.x;
   for (int c = threadIdx.x; c < H; c += 256) {
     float s = 0.f;
-    for (int r = 0; r < top; ++r) s += wts[(long)t * top + r] * y[(long)pair_row[(long)t * top + r] * H + c];
+    for (int r = 0; r < top; ++r) {
+      const int row = pair_row[(long)t * top + r];
+      s += wts[(long)t * top + r] * (row >= 0 ? y[(long)row * H + c] : (x ? x[(long)t * ldx + c] : 0.f));
+    }
     out[(long)t * ldo + c] = s;
   }
 }
@@ -336,10 +365,10 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ ou
 }  // namespace dlia
 
 extern "C" void dlia_moe_route(int* sel, float* wts, const float* logits, long ld, int T, int E, int top, int groups, int keep,
-                               float scale, hipStream_t stream) {
+                               float scale, const float* corr, int softmax, int group_rank, int renorm, hipStream_t stream) {
   if (T <= 0) return;
   hipLaunchKernelGGL(dlia::moe_route_kernel, dim3((T + 63) / 64), dim3(64), 0, stream, sel, wts, logits, ld, T, E, top, groups,
-                     keep, scale);
+                     keep, scale, corr, softmax, group_rank, renorm);
 }
 
 extern "C" void dlia_moe_plan(int* tiles, int* row_tok, int* pair_row, const int* sel, int pairs, int top, int E, int max_rows,
@@ -402,7 +431,7 @@ extern "C" void dlia_moe_down(float* y, const void* act, const void* wd, int f32
 }
 
 extern "C" void dlia_moe_combine(float* out, const float* y, const int* pair_row, const float* wts, int T, int H, int top, long ldo,
-                                 hipStream_t stream) {
+                                 const float* x, long ldx, hipStream_t stream) {
   if (T <= 0) return;
-  hipLaunchKernelGGL(dlia::moe_combine_kernel, dim3(T), dim3(256), 0, stream, out, y, pair_row, wts, H, top, ldo);
+  hipLaunchKernelGGL(dlia::moe_combine_kernel, dim3(T), dim3(256), 0, stream, out, y, pair_row, wts, H, top, ldo, x, ldx);
 }

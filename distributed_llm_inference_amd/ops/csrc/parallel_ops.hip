@@ -15,6 +15,9 @@
 //                   the sequence's first tokens, scores through cap tanh(s / cap); with two maps per head both are
 //                   walked at once over the shared values and combined as rms(a1 - lam a2) (1 - diff) sigmoid(gate).
 //                   Keys are rows of any length (a map is a slice of the row), values may be a slice of the key rows.
+//                   The key cache may have fewer heads than the value cache (one row of all key heads for queries that carry
+//                   a mix of heads); `chunk` > 0 hides the keys of other chunks of that many positions; `sink` [H] adds
+//                   exp(sink[h]) to the softmax's denominator.
 //   rglru_scan      S <- a S + sqrt(1 - a^2) i u per channel with a = exp(-c r), r and i sigmoids of the block gates;
 //                   read-out S * gelu_tanh(y). Long portions are cut into stretches that are scanned side by side and
 //                   joined through the stretches' (decay product, end value) pairs: inside a workgroup through LDS, or,
@@ -180,12 +183,12 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
     const T* __restrict__ vcache, int v_row, int v_off, const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
     const int* __restrict__ block_table, int items, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
     float scale, int window, int keep_first, float softcap, float lam, float post, float eps, const float* __restrict__ gate,
-    long ldg, int vec) {
+    long ldg, int vec, int Gk, int chunk, const float* __restrict__ sink) {
   __shared__ float qs[4][kMultiMaxQ];
   const int wave = threadIdx.x >> 6, lane = lane_id();
   const int item = blockIdx.x * 4 + wave;
   if (item >= items) return;
-  const int t = item / H, h = item % H, g = h / (H / G);
+  const int t = item / H, h = item % H, g = h / (H / G), gk = h / (H / Gk);
   const int pos = tok_pos[t], slot = tok_seq[t];
   OT* orow = out + (long)t * ldo + (long)h * dv;
   const bool live = slot >= 0 && slot < table_rows && pos >= 0 && pos / kParBlock < max_blocks;
@@ -197,7 +200,8 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
   for (int i = lane; i < MAPS * d; i += 64) qs[wave][i] = qrow[i] * scale;
   __builtin_amdgcn_wave_barrier();
   const int* table = block_table + (long)slot * max_blocks;
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  if (chunk > 0) lo = max(lo, pos / chunk * chunk);                             // the query's own chunk only
   const int kept = (window > 0 && keep_first > 0) ? min(keep_first, lo) : 0;    // keys [0, kept) in front of the window
   float m[MAPS], l[MAPS], acc[MAPS][kMultiMaxDV / 64];
 #pragma unroll
@@ -221,7 +225,7 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
       for (int a = 0; a < MAPS; ++a) {
         s[a] = -INFINITY;
         if (valid) {
-          const T* krow = kcache + (((long)blk * G + g) * kParBlock + (j % kParBlock)) * k_row + a * d;
+          const T* krow = kcache + (((long)blk * Gk + gk) * kParBlock + (j % kParBlock)) * k_row + a * d;
           float dot = dot_row(qs[wave] + a * d, krow, d, vec != 0);
           if (softcap > 0.f) dot = softcap * tanhf(dot * inv_cap);
           s[a] = dot;
@@ -258,6 +262,11 @@ __global__ __launch_bounds__(256) void multi_attention_kernel(
           }
       }
     }
+  }
+  if (sink) {
+    // one more term in the denominator: a key of score sink[h] that has no value
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) l[a] = m[a] == -INFINITY ? 1.f : l[a] + expf(sink[h] - m[a]);
   }
   float o[kMultiMaxDV / 64];
   const float i0 = l[0] > 0.f ? 1.f / l[0] : 0.f;
@@ -304,7 +313,7 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
     const bf16* __restrict__ vt, const int* __restrict__ q_start, const int* __restrict__ ctx, const int* __restrict__ slots,
     const int* __restrict__ block_table, int tiles_per_seq, int max_blocks, int num_blocks, int table_rows, int H, int G, int d,
     int dv, float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
-    const float* __restrict__ gate, long ldg, float* __restrict__ part) {
+    const float* __restrict__ gate, long ldg, float* __restrict__ part, int Gk, int chunk, const float* __restrict__ sink) {
   extern __shared__ __attribute__((aligned(16))) bf16 qs_all[];        // per wave [16][MAPS * d + 8]
   // Rows of a wave's tile. Prompt portions: 16 consecutive tokens of one head; the waves of a workgroup take neighbouring heads
   // (those of one key / value head first), so the key and value fragments they all read come from L1 after the first.
@@ -353,7 +362,10 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
     for (int c = 0; c < DVT; ++c) o[a][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
   const float inv_cap = softcap > 0.f ? 1.f / softcap : 0.f;
-  const int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  int lo_first = (window > 0 && pos_first - window + 1 > 0) ? pos_first - window + 1 : 0;
+  if (chunk > 0) lo_first = max(lo_first, pos_first / chunk * chunk);     // (the first row's chunk starts lowest)
+  const int chunk_lo = chunk > 0 ? qpos / chunk * chunk : 0;
+  const int gk = Gk == G ? g : 0;                                         // (the key cache has G heads or one)
   const int kb_lo = lo_first / kParBlock, kb_hi = min(pos_last / kParBlock, max_blocks - 1);
   const int kept = (window > 0 && keep_first > 0) ? min(keep_first, lo_first) : 0;
   const int kb_kept = kept > 0 ? min((kept - 1) / kParBlock, kb_lo - 1) : -1;      // blocks [0, kb_kept] hold kept tokens only
@@ -368,7 +380,7 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
     f32x4 s[MAPS][2];
 #pragma unroll
     for (int a = 0; a < MAPS; ++a) s[a][0] = s[a][1] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const bf16* kbase = kcache + ((long)blk * G + g) * kParBlock * k_row;
+    const bf16* kbase = kcache + ((long)blk * Gk + gk) * kParBlock * k_row;
     for (int k0 = 0; k0 < d; k0 += 32 * KS) {
       u32x4 ak[MAPS][KS][2];          // KS k-steps of key fragments in flight at once
 #pragma unroll
@@ -416,7 +428,7 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const int j = kb * kParBlock + (i >> 2) * 16 + kq * 4 + (i & 3);
-        const bool vis = qvalid && j <= qpos && (window <= 0 || qpos - j < window || j < keep_first);
+        const bool vis = qvalid && j <= qpos && j >= chunk_lo && (window <= 0 || qpos - j < window || j < keep_first);
         float x = s[a][i >> 2][i & 3] * scale;
         if (softcap > 0.f) x = softcap * tanhf(x * inv_cap);
         sv[i] = vis ? x : -INFINITY;
@@ -492,6 +504,11 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
     }
     return;
   }
+  if (sink && qvalid) {
+    const float sk = sink[h];
+#pragma unroll
+    for (int a = 0; a < MAPS; ++a) lsum[a] = m[a] == -INFINITY ? 1.f : lsum[a] + expf(sk - m[a]);
+  }
 #pragma unroll
   for (int a = 0; a < MAPS; ++a) inv[a] = lsum[a] > 0.f ? 1.f / lsum[a] : 0.f;
   float mul = inv[0];
@@ -533,7 +550,7 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
 template <int MAPS>
 __global__ __launch_bounds__(256) void tile_merge_kernel(bf16* __restrict__ out, long ldo, const float* __restrict__ part, int items,
                                                          int H, int dv, int nz, float lam, float post, float eps,
-                                                         const float* __restrict__ gate, long ldg) {
+                                                         const float* __restrict__ gate, long ldg, const float* __restrict__ sink) {
   const int item = blockIdx.x * 4 + (threadIdx.x >> 6), lane = lane_id();
   if (item >= items) return;
   const int t = item / H, h = item % H;
@@ -555,6 +572,7 @@ __global__ __launch_bounds__(256) void tile_merge_kernel(bf16* __restrict__ out,
 #pragma unroll
       for (int c = 0; c < kMultiMaxDV / 64; ++c) { const int col = c * 64 + lane; if (col < dv) o[a][c] += pz[col] * w; }
     }
+    if (sink) L = M == -INFINITY ? 1.f : L + expf(sink[h] - M);
     const float inv = L > 0.f ? 1.f / L : 0.f;
 #pragma unroll
     for (int c = 0; c < kMultiMaxDV / 64; ++c) o[a][c] *= inv;
@@ -759,22 +777,23 @@ static void launch_multi(int maps, dim3 grid, hipStream_t stream, void* out, lon
                          const void* kc, int k_row, const void* vc, int v_row, int v_off, const int* tok_pos, const int* tok_seq,
                          const int* table, int items, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
                          float scale, int window, int keep_first, float softcap, float lam, float post, float eps,
-                         const float* gate, long ldg, int vec) {
+                         const float* gate, long ldg, int vec, int Gk, int chunk, const float* sink) {
   if (maps == 2)
     hipLaunchKernelGGL((multi_attention_kernel<T, OT, 2>), grid, dim3(256), 0, stream, (OT*)out, ldo, q, ldq, q_head, (const T*)kc,
                        k_row, (const T*)vc, v_row, v_off, tok_pos, tok_seq, table, items, max_blocks, num_blocks, table_rows, H, G,
-                       d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, vec);
+                       d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, vec, Gk, chunk, sink);
   else
     hipLaunchKernelGGL((multi_attention_kernel<T, OT, 1>), grid, dim3(256), 0, stream, (OT*)out, ldo, q, ldq, q_head, (const T*)kc,
                        k_row, (const T*)vc, v_row, v_off, tok_pos, tok_seq, table, items, max_blocks, num_blocks, table_rows, H, G,
-                       d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, vec);
+                       d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, vec, Gk, chunk, sink);
 }
 
 extern "C" void dlia_multi_attention(void* out, long ldo, const float* q, long ldq, int q_head, const void* kcache, int k_row,
                                      const void* vcache, int v_row, int v_off, int f32, const int* tok_pos, const int* tok_seq,
                                      const int* block_table, int T, int max_blocks, int num_blocks, int table_rows, int H, int G,
                                      int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam,
-                                     float post, float eps, const float* gate, long ldg, hipStream_t stream) {
+                                     float post, float eps, const float* gate, long ldg, int Gk, int chunk, const float* sink,
+                                     hipStream_t stream) {
   const int items = T * H;
   if (items <= 0) return;
   const dim3 grid((items + 3) / 4);
@@ -783,11 +802,11 @@ extern "C" void dlia_multi_attention(void* out, long ldo, const float* q, long l
   if (f32)
     launch_multi<float, float>(maps, grid, stream, out, ldo, q, ldq, q_head, kcache, k_row, vcache, v_row, v_off, tok_pos, tok_seq,
                                block_table, items, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first,
-                               softcap, lam, post, eps, gate, ldg, vec);
+                               softcap, lam, post, eps, gate, ldg, vec, Gk, chunk, sink);
   else
     launch_multi<bf16, bf16>(maps, grid, stream, out, ldo, q, ldq, q_head, kcache, k_row, vcache, v_row, v_off, tok_pos, tok_seq,
                              block_table, items, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first,
-                             softcap, lam, post, eps, gate, ldg, vec);
+                             softcap, lam, post, eps, gate, ldg, vec, Gk, chunk, sink);
 }
 
 extern "C" long dlia_rglru_scan_ws_floats(int rows, int B, int W) { return ((long)rows / kScanStretch + 2 * B + 2) * W * 2; }
@@ -848,8 +867,10 @@ extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq,
                                    const void* vt, const int* q_start, const int* ctx, const int* slots, const int* block_table,
                                    int B, int max_q, int max_blocks, int num_blocks, int table_rows, int H, int G, int d, int dv,
                                    int maps, float scale, int window, int keep_first, float softcap, float lam, float post,
-                                   float eps, const float* gate, long ldg, float* part, long part_floats, hipStream_t stream) {
+                                   float eps, const float* gate, long ldg, float* part, long part_floats, int Gk, int chunk,
+                                   const float* sink, hipStream_t stream) {
   if (B <= 0 || max_q <= 0) return 0;
+  if (Gk != G && Gk != 1) return 1;
   if (d % 8 || k_row % 8 || q_head % 8 || ldq % 8 || maps * d > 1024 || dv > 512 || (maps != 1 && maps != 2)) return 1;
   const bool head_rows = max_q == 1;
   const int tiles = (max_q + 15) / 16, group = H / G;
@@ -867,12 +888,12 @@ extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq,
     if (head_rows)                                                                                                               \
       hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, true, KS>), grid, dim3(64), lds, stream, (bf16*)out, ldo, (const bf16*)q, ldq, \
                          q_head, (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, tiles, max_blocks,   \
-                         num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, part);  \
+                         num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps, gate, ldg, part, Gk, chunk, sink);  \
     else                                                                                                                         \
       hipLaunchKernelGGL((tile_attention_kernel<MAPS, DVT, false, KS>), grid, dim3(64 * nw), lds, stream, (bf16*)out, ldo,              \
                          (const bf16*)q, ldq, q_head, (const bf16*)kcache, k_row, (const bf16*)vt, q_start, ctx, slots, block_table, \
                          tiles, max_blocks, num_blocks, table_rows, H, G, d, dv, scale, window, keep_first, softcap, lam, post, eps,  \
-                         gate, ldg, part);                                                                                       \
+                         gate, ldg, part, Gk, chunk, sink);                                                                      \
   } while (0)
   // (a map's whole key row in flight when it is long and the registers allow: one wait per block instead of four)
 #define DLIA_TILE(MAPS, DVT)                                            \
@@ -889,10 +910,10 @@ extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq,
     const int items = B * H;
     if (maps == 2)
       hipLaunchKernelGGL(tile_merge_kernel<2>, dim3((items + 3) / 4), dim3(256), 0, stream, (bf16*)out, ldo, part, items, H, dv, nz, lam,
-                         post, eps, gate, ldg);
+                         post, eps, gate, ldg, sink);
     else
       hipLaunchKernelGGL(tile_merge_kernel<1>, dim3((items + 3) / 4), dim3(256), 0, stream, (bf16*)out, ldo, part, items, H, dv, nz, lam,
-                         post, eps, gate, ldg);
+                         post, eps, gate, ldg, sink);
   }
 #undef DLIA_TILE
 #undef DLIA_TILE_KS
