@@ -88,6 +88,9 @@ def parse():
     ap.add_argument("--parallel-compare", action="store_true",
                     help="instead of the serving benchmark: prefill and decode throughput of a Tezesun stack beside the Letarax stack "
                          "of equal size on one GPU (bench/hybrid_compare.py), one JSON line per size")
+    ap.add_argument("--postnorm-compare", action="store_true",
+                    help="instead of the serving benchmark: prefill and decode throughput of a Zovozen stack beside the Nufapel stack "
+                         "of equal size on one GPU (bench/hybrid_compare.py), one JSON line per size")
     ap.add_argument("--hybrid-sizes", default="", help="with --hybrid-compare: comma-separated size names (default: all)")
     ap.add_argument("--preflight", action="store_true",
                     help="no model: report devices, peer access and RCCL, open + warm + time + close every hop, exit")
@@ -396,11 +399,11 @@ def preflight(a, world: int, emit=print) -> int:
 
 def main():
     a = parse()
-    if a.hybrid_compare or a.gated_compare or a.parallel_compare:
+    if a.hybrid_compare or a.gated_compare or a.parallel_compare or a.postnorm_compare:
         sys.path.insert(0, os.path.join(ROOT, "bench"))
         import hybrid_compare
         raise SystemExit(hybrid_compare.main([x for x in a.hybrid_sizes.split(",") if x] or None, gated=a.gated_compare,
-                                                parallel=a.parallel_compare))
+                                                parallel=a.parallel_compare, postnorm=a.postnorm_compare))
     env_world = os.environ.get("WORLD_SIZE")
     if env_world is None and a.gpus > 1:
         # no launcher: this process becomes one (it never touches a GPU; nothing below runs in it)

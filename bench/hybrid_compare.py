@@ -1,6 +1,7 @@
 """Prefill and decode throughput of a Letarax stack beside a Llama stack of equal size (`bench.py --hybrid-compare`), of a
-Nufapel stack beside the Letarax stack of equal size (`bench.py --gated-compare`), and of a Tezesun stack beside the
-Letarax stack of equal size (`bench.py --parallel-compare`).
+Nufapel stack beside the Letarax stack of equal size (`bench.py --gated-compare`), of a Tezesun stack beside the
+Letarax stack of equal size (`bench.py --parallel-compare`), and of a Zovozen stack beside the Nufapel stack of equal size
+(`bench.py --postnorm-compare`).
 
 Both models get random weights and the same width, head counts, head size, feed-forward width, depth and
 vocabulary; the Letarax stack has three attention layers (windowed, with the sink and value mixing) to one delta-rule
@@ -35,6 +36,14 @@ def parallel_specs(name: str):
     attention over the paged cache beside recurrent layers with slot-resident state)."""
     from distributed_llm_inference_amd.models.spec import BUILTIN_SPECS
     return BUILTIN_SPECS[f"tezesun-{name}"], BUILTIN_SPECS[f"letarax-{name}"]
+
+
+def postnorm_specs(name: str):
+    """The Zovozen stack of a size (attention with mixed heads, chunked mask and sink beside a matrix memory; routed and dense
+    feed-forwards alternating) beside the closest existing design of the same width, heads, head size, feed-forward and
+    depth: the Nufapel stack (attention beside a matrix memory in three layers of four, routed feed-forwards)."""
+    from distributed_llm_inference_amd.models.spec import BUILTIN_SPECS
+    return BUILTIN_SPECS[f"zovozen-{name}"], BUILTIN_SPECS[f"nufapel-{name}"]
 
 
 def specs(name: str):
@@ -101,15 +110,15 @@ def time_decode(ex, rows: int, ctx: int, iters: int) -> float:
     return e0.elapsed_time(e1) / 1e3 / iters
 
 
-def main(sizes=None, iters: int = 8, out=sys.stdout, gated: bool = False, parallel: bool = False) -> int:
+def main(sizes=None, iters: int = 8, out=sys.stdout, gated: bool = False, parallel: bool = False, postnorm: bool = False) -> int:
     import gc
     import torch
     rows, ctx, plen = 64, 1024, 2048
     for name in (sizes or list(SIZES)):
-        rec = {"metric": "tezesun_vs_letarax_tokens_per_s" if parallel else "nufapel_vs_letarax_tokens_per_s" if gated else "letarax_vs_llama_tokens_per_s", "size": name, "dtype": "bf16", "data": "synthetic", "weights": "random",
+        rec = {"metric": "zovozen_vs_nufapel_tokens_per_s" if postnorm else "tezesun_vs_letarax_tokens_per_s" if parallel else "nufapel_vs_letarax_tokens_per_s" if gated else "letarax_vs_llama_tokens_per_s", "size": name, "dtype": "bf16", "data": "synthetic", "weights": "random",
                "config": dict(zip(("width", "heads", "kv_heads", "head_dim", "ff", "layers", "window"), SIZES[name])),
                "prefill": {"prompts": 1, "tokens": plen}, "decode": {"rows": rows, "context": ctx}}
-        for spec in (parallel_specs(name) if parallel else gated_specs(name) if gated else specs(name)):
+        for spec in (postnorm_specs(name) if postnorm else parallel_specs(name) if parallel else gated_specs(name) if gated else specs(name)):
             t0 = time.perf_counter()
             ex = build(spec, rows, plen, max(plen, ctx + 256))
             tp = time_prefill(ex, 1, plen, iters)
@@ -123,7 +132,7 @@ def main(sizes=None, iters: int = 8, out=sys.stdout, gated: bool = False, parall
             del ex
             gc.collect()
             torch.cuda.empty_cache()
-        new, old = ("tezesun", "letarax") if parallel else ("nufapel", "letarax") if gated else ("letarax", "llama")
+        new, old = ("zovozen", "nufapel") if postnorm else ("tezesun", "letarax") if parallel else ("nufapel", "letarax") if gated else ("letarax", "llama")
         rec["prefill_ratio"] = round(rec[new]["prefill_tok_s"] / rec[old]["prefill_tok_s"], 3)
         rec["decode_ratio"] = round(rec[new]["decode_tok_s"] / rec[old]["decode_tok_s"], 3)
         out.write(json.dumps(rec) + "\n")

@@ -119,7 +119,7 @@ void mix_prep(const Tensor& z, int64_t H, int64_t G, int64_t d, int64_t dv, OptT
                                kcache.data_ptr(), (int)Gk, vcache.data_ptr(), v_t ? 1 : 0, is_f32(kcache), tok_pos.data_ptr<int>(),
                                tok_seq.data_ptr<int>(), block_table.data_ptr<int>(), (int)block_table.size(1), (int)kcache.size(0),
                                (int)block_table.size(0), cur_stream());
-  DLIA_CHECK(rc == 0, "mix_prep: q and k of one token ((H + G) d floats) must fit a workgroup's 64 KiB of LDS");
+  DLIA_CHECK(rc == 0, "mix_prep: q and k of one token and the mix ((H + G) d + H H floats) must fit a workgroup's 64 KiB of LDS");
 }
 
 }  // namespace

@@ -324,13 +324,17 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
   const int group = H / G;
   const int b = blockIdx.x / tiles_per_seq, ti = blockIdx.x % tiles_per_seq;
   const int t0 = q_start[b], n = q_start[b + 1] - t0, c0 = ctx[b], slot = slots[b];
+  // (HEADROWS over ONE key row for all heads, Gk == 1 < G: a tile's rows are 16 consecutive heads whatever their value head, so
+  // the keys are read once per 16 heads; the value product then runs once per value head of the tile, on the weights of that
+  // head's rows)
+  const bool all_heads = HEADROWS && Gk == 1 && G > 1;
   int h, g, r0, nrows;
   if constexpr (HEADROWS) {
     const int gt = (group + 15) / 16;
-    g = blockIdx.y / gt;
-    h = g * group + (blockIdx.y % gt) * 16;                             // head of row 0
+    g = all_heads ? 0 : blockIdx.y / gt;
+    h = all_heads ? blockIdx.y * 16 : g * group + (blockIdx.y % gt) * 16;   // head of row 0
     r0 = 0;
-    nrows = n > 0 ? min(16, group - (blockIdx.y % gt) * 16) : 0;
+    nrows = n <= 0 ? 0 : all_heads ? min(16, H - h) : min(16, group - (blockIdx.y % gt) * 16);
   } else {
     h = blockIdx.y * (blockDim.x >> 6) + wave;
     g = h < H ? h / group : 0;
@@ -366,6 +370,8 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
   if (chunk > 0) lo_first = max(lo_first, pos_first / chunk * chunk);     // (the first row's chunk starts lowest)
   const int chunk_lo = chunk > 0 ? qpos / chunk * chunk : 0;
   const int gk = Gk == G ? g : 0;                                         // (the key cache has G heads or one)
+  const int g_lo = all_heads ? h / group : g, g_hi = all_heads ? (h + nrows - 1) / group : g;
+  const int my_g = all_heads ? min(h + r16, H - 1) / group : g;
   const int kb_lo = lo_first / kParBlock, kb_hi = min(pos_last / kParBlock, max_blocks - 1);
   const int kept = (window > 0 && keep_first > 0) ? min(keep_first, lo_first) : 0;
   const int kb_kept = kept > 0 ? min((kept - 1) / kParBlock, kb_lo - 1) : -1;      // blocks [0, kb_kept] hold kept tokens only
@@ -406,7 +412,7 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
     // memory overlaps the softmax. (With more accumulators the registers do not hold them as well: fragment by fragment then.)
     constexpr bool AHEAD = MAPS * DVT <= 16;
     constexpr int VB = DVT > 8 ? 8 : DVT;
-    const bf16* vbase = vt + ((long)blk * G + g) * dv * kParBlock + (long)r16 * kParBlock + kq * 4;
+    const bf16* vbase = vt + ((long)blk * G + g_lo) * dv * kParBlock + (long)r16 * kParBlock + kq * 4;
     u32x4 av[VB];
     auto load_values = [&](int c0) {
 #pragma unroll
@@ -452,30 +458,39 @@ __global__ __launch_bounds__(256) void tile_attention_kernel(
       for (int c = 0; c < DVT; ++c) o[a][c] *= corr;
       pf[a] = pack8(p);
     }
-    if constexpr (AHEAD) {
+    for (int gv = g_lo; gv <= g_hi; ++gv) {
+      u32x4 pm[MAPS];                   // the weights of the rows whose values are head gv's
 #pragma unroll
-      for (int c0 = 0; c0 < DVT; c0 += VB) {
-        if (c0 * 16 >= dv) break;
-        if (c0 > 0) load_values(c0);
-#pragma unroll
-        for (int j = 0; j < VB; ++j) {
-          if ((c0 + j) * 16 >= dv) break;
-#pragma unroll
-          for (int a = 0; a < MAPS; ++a) o[a][c0 + j] = mfma16(av[j], pf[a], o[a][c0 + j]);
-        }
+      for (int a = 0; a < MAPS; ++a) pm[a] = my_g == gv ? pf[a] : zero;
+      if (gv > g_lo) {
+        vbase += (long)dv * kParBlock;
+        if constexpr (AHEAD) load_values(0);
       }
-    } else {
+      if constexpr (AHEAD) {
 #pragma unroll
-      for (int c = 0; c < DVT; ++c) {
-        if (c * 16 >= dv) break;
-        u32x4 v1 = zero;
-        if (c * 16 + r16 < dv) {
-          const u32x2 lo = *reinterpret_cast<const u32x2*>(vbase + (long)c * 16 * kParBlock);
-          const u32x2 hi = *reinterpret_cast<const u32x2*>(vbase + (long)c * 16 * kParBlock + 16);
-          v1 = u32x4{lo.x, lo.y, hi.x, hi.y};
+        for (int c0 = 0; c0 < DVT; c0 += VB) {
+          if (c0 * 16 >= dv) break;
+          if (c0 > 0) load_values(c0);
+#pragma unroll
+          for (int j = 0; j < VB; ++j) {
+            if ((c0 + j) * 16 >= dv) break;
+#pragma unroll
+            for (int a = 0; a < MAPS; ++a) o[a][c0 + j] = mfma16(av[j], pm[a], o[a][c0 + j]);
+          }
         }
+      } else {
 #pragma unroll
-        for (int a = 0; a < MAPS; ++a) o[a][c] = mfma16(v1, pf[a], o[a][c]);
+        for (int c = 0; c < DVT; ++c) {
+          if (c * 16 >= dv) break;
+          u32x4 v1 = zero;
+          if (c * 16 + r16 < dv) {
+            const u32x2 lo = *reinterpret_cast<const u32x2*>(vbase + (long)c * 16 * kParBlock);
+            const u32x2 hi = *reinterpret_cast<const u32x2*>(vbase + (long)c * 16 * kParBlock + 16);
+            v1 = u32x4{lo.x, lo.y, hi.x, hi.y};
+          }
+#pragma unroll
+          for (int a = 0; a < MAPS; ++a) o[a][c] = mfma16(v1, pm[a], o[a][c]);
+        }
       }
     }
   }
@@ -878,8 +893,10 @@ extern "C" int dlia_tile_attention(void* out, long ldo, const void* q, long ldq,
   const size_t qtile = (size_t)16 * (maps * d + 8) * sizeof(bf16);
   int nw = head_rows ? 1 : (group % 4 == 0 || G == 1) && H >= 4 ? 4 : (group % 2 == 0 && H >= 2 ? 2 : 1);
   while (nw > 1 && nw * qtile > 65536) nw >>= 1;           // (a workgroup's LDS)
-  const int nz = head_rows ? dlia_tile_attention_splits(B, H, G) : 1;
-  const dim3 grid(B * tiles, head_rows ? G * ((group + 15) / 16) : (H + nw - 1) / nw, nz);
+  // (single tokens over one key row for all heads: tiles of 16 consecutive heads, see the kernel)
+  const bool all_heads = head_rows && Gk == 1 && G > 1;
+  const int nz = head_rows ? dlia_tile_attention_splits(B, H, all_heads ? 1 : G) : 1;
+  const dim3 grid(B * tiles, all_heads ? (H + 15) / 16 : head_rows ? G * ((group + 15) / 16) : (H + nw - 1) / nw, nz);
   const size_t lds = nw * qtile;
   if (lds > 65536) return 1;
   if (head_rows && (!part || part_floats < (long)B * H * maps * nz * (dv + 2))) return 2;

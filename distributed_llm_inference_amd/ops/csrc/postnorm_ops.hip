@@ -61,6 +61,9 @@ __global__ __launch_bounds__(kPostThreads) void mix_prep_kernel(
   float* qs = sm;
   float* ks = sm + qn;
   float* scratch = ks + kn;
+  float* ms = scratch + 16;             // the head mix [H, H]
+  if (mix)
+    for (int i = threadIdx.x; i < H * H; i += kPostThreads) ms[i] = mix[i];
   const int t = blockIdx.x;
   const int pos = tok_pos[t], slot = tok_seq[t];
   const float* zr = z + (long)t * ldz;
@@ -91,12 +94,24 @@ __global__ __launch_bounds__(kPostThreads) void mix_prep_kernel(
   if (q_out) {
     QT* qo = q_out + (long)t * ldqo;
     if (mix) {
+      // A thread takes one entry (key head c, place i) of the query rows of ALL heads: the group's queries at that place are
+      // read once, the mix comes from LDS (every lane of a wave reads the same address: a broadcast), and a wave's stores
+      // cover consecutive entries of one head's row.
       const int group = H / G, row = G * d;
-      for (int idx = threadIdx.x; idx < H * row; idx += kPostThreads) {
-        const int h = idx / row, c = (idx % row) / d, i = idx % d;
-        float acc = 0.f;
-        for (int g = c * group; g < (c + 1) * group; ++g) acc += mix[h * H + g] * qs[g * d + i];
-        qo[idx] = (QT)acc;
+      for (int e = threadIdx.x; e < row; e += kPostThreads) {
+        const int c = e / d, i = e % d;
+        for (int h0 = 0; h0 < H; h0 += 8) {
+          float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+          for (int j = 0; j < group; ++j) {
+            const float qv = qs[(c * group + j) * d + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+              if (h0 + u < H) acc[u] += ms[(h0 + u) * H + c * group + j] * qv;
+          }
+#pragma unroll
+          for (int u = 0; u < 8; ++u)
+            if (h0 + u < H) qo[(long)(h0 + u) * row + e] = (QT)acc[u];
+        }
       }
     } else {
       for (int i = threadIdx.x; i < qn; i += kPostThreads) qo[i] = (QT)qs[i];
@@ -149,7 +164,7 @@ extern "C" int dlia_mix_prep(const float* z, long ldz, int T, int H, int G, int 
                              const int* tok_seq, const int* block_table, int max_blocks, int num_blocks, int table_rows,
                              hipStream_t stream) {
   if (T <= 0) return 0;
-  const size_t lds = ((size_t)(H + G) * d + 16) * sizeof(float);
+  const size_t lds = ((size_t)(H + G) * d + 16 + (mix ? (size_t)H * H : 0)) * sizeof(float);
   if (lds > 65536) return 1;
 #define DLIA_PREP(CT, QT)                                                                                                      \
   hipLaunchKernelGGL((dlia::mix_prep_kernel<CT, QT>), dim3(T), dim3(dlia::kPostThreads), lds, stream, z, ldz, H, G, d, dv, qw, kw, eps, \

@@ -155,7 +155,7 @@ def _prep_and_attend(K, dev, dtype, tile, H, G, d, dv, chunk, dims, mixed, z_all
         qf = torch.zeros(T, H * kd, device=dev, dtype=dtype if tile else torch.float32)
         K.mix_prep(z, H, G, d, dv, f(P["q.norm"]), f(P["k.norm"]), eps, dims, cos, sin, True, mix, qf, kc, vc, tile, tok_pos, tok_seq, table)
         if tile:
-            part = torch.zeros(int(K.tile_attention_part_floats(len(step), H, G, dv, 1)), device=dev)
+            part = torch.zeros(int(K.tile_attention_part_floats(len(step), H, 1 if mixed else G, dv, 1)), device=dev)   # (one key row for all heads: tiles of 16 heads)
             K.tile_attention(out, qf, kd, kc, vc, q_start, ctx, slots, table, max(n for _, _, n in step), H, kd, dv, 1, 1.0 if mixed else scale,
                              0, 0, 0.0, 0.0, 1.0, eps, gt, part, chunk, f(P["sink"]))
         else:
