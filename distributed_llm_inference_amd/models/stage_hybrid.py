@@ -44,9 +44,10 @@ Stacks that norm their sublayers' OUTPUTS only (`spec.post_norm`: the sublayers 
 
     x (fp32, and in the GEMMs' type) -> ONE input GEMM (all projections of both mixers, biases in the epilogue)
              -> [ q / k norms over the whole projection + rotation + unit values + the head mix folded into the query
-                  + cache write (one kernel) -> attention with chunked mask, learned sink and output gate -> o GEMM
-                  beside   matrix memory (exponential gates) -> per-head norm * weight * gate -> o GEMM ]
-             -> x += rms(a left + b right) w, and x in the GEMMs' type (one kernel)
+                  + cache write (one kernel) -> attention with chunked mask, learned sink and output gate
+                  beside   matrix memory (exponential gates) -> per-head norm * weight * gate ]
+             -> ONE output GEMM over both branches' rows (the branch weights' ratio rides in the memory's norm weight)
+             -> x += rms(a y) w, and x in the GEMMs' type (one kernel)
              -> [ up GEMM -> squared relu -> down GEMM
                 | router + shared gate / up GEMM -> route -> plan -> the experts' GEMMs over sorted rows -> weighted sum with
                   the identity experts' share of x;  silu(gate) * up -> shared down GEMM ]
@@ -903,8 +904,14 @@ class HybridGpuStage(GpuStage):
             if a.proj_bias:
                 b_in[:l["b_qkv"].numel()] = f32(l["b_qkv"])
             self._matrix(p, "w_in", w_in, b_in)
-            self._matrix(p, "w_o", mat(l["w_o"]), f32(l["b_o"]) if a.proj_bias else None)
-            self._matrix(p, "w_o_r", mat(l["w_o_r"]), None)
+            # a * (W_l m_l + b) + b' * W_r m_r = a * ([W_l | W_r] [m_l | (b' / a) m_r] + b): ONE output GEMM over both branches' mixed
+            # rows, the ratio of the branch weights carried by the memory's norm weight (fp32), `a` applied where the sum is normed
+            sa, sb = ls.branch_scales or (1.0, 1.0)
+            w_l, b_l = mat(l["w_o"]), f32(l["b_o"]) if a.proj_bias else None
+            if sa == 0.0:
+                w_l, b_l, sa, sb = torch.zeros_like(w_l), None, 1.0, sb
+            self._matrix(p, "w_o", torch.cat([w_l, mat(l["w_o_r"])], dim=1).contiguous(), b_l)
+            p["out_scale"] = float(sa)
             p["q_norm_w"], p["k_norm_w"] = (f32(l["q_norm_w"]), f32(l["k_norm_w"])) if a.qk_norm else (None, None)
             # score_h = sum_g talk[h, g] temp[g] scale (q_g . k): the mix, the temperatures and the scale are one matrix
             p["mix"] = None
@@ -921,7 +928,7 @@ class HybridGpuStage(GpuStage):
                 p["cos"], p["sin"] = tables[key]
             else:
                 p["cos"] = p["sin"] = None
-            p["b_if"], p["o_norm_w"] = f32(l["b_if"]), f32(l["o_norm_w"])
+            p["b_if"], p["o_norm_w"] = f32(l["b_if"]), (f32(l["o_norm_w"]) * (sb / sa)).contiguous()
             if ls.has_ff:
                 p["ln2_w"] = f32(l["ln2_w"])
             if ls.moe is not None:
@@ -953,8 +960,8 @@ class HybridGpuStage(GpuStage):
         for ls, p, tile in zip(self.specs, self.layers, self._tile):
             a, b = ls.branches
             zc, qc = max(zc, self._cols(p, "w_in")), max(qc, a.heads * self._query_row(a))
-            mc, m2, oc = max(mc, a.heads * a.vdim), max(m2, b.heads * b.vdim), max(oc, b.heads * (b.vdim + 2))
-            yc = max(yc, self._cols(p, "w_o"), self._cols(p, "w_o_r"))
+            mc, oc = max(mc, a.heads * a.vdim + b.heads * b.vdim), max(oc, b.heads * (b.vdim + 2))
+            yc = max(yc, self._cols(p, "w_o"))
             if tile:
                 # (with the mix folded into the query a tile holds 16 heads of any value head: the splits of one key / value head)
                 gs = 1 if (a.head_mix or a.head_temp) else a.kv_heads
@@ -978,7 +985,7 @@ class HybridGpuStage(GpuStage):
         return SimpleNamespace(
             h=torch.zeros(rows, H, device=dev), xn=torch.zeros(rows, H, device=dev, dtype=at), z=z(rows * zc),
             qf=z(rows * qc, at if any(self._tile) else torch.float32), qf32=z(rows * qc if not all(self._tile) else 1),
-            o=z(rows * oc), mixed=z(rows * mc, at), mixed2=z(rows * m2, at), ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2),
+            o=z(rows * oc), mixed=z(rows * mc, at), ya=z(rows * yc), yb=z(rows * yc), z2=z(rows * z2),
             act=z(rows * ac, at), acts=z(rows * sc, at), sel=z(pairs, i32), wts=z(pairs), pair_row=z(pairs, i32), tiles=z(1 + tiles, i32),
             row_tok=z(32 * tiles, i32), eact=z(32 * tiles * ef, at), ey=z(32 * tiles * H), part=z(part), ws=z(ws_floats + 4096),
             head_x=torch.zeros(B, H, device=dev, dtype=at), logits=torch.zeros(B, self.vocab_pad, device=dev), cmax=None, guided=False)
@@ -1005,7 +1012,8 @@ class HybridGpuStage(GpuStage):
             kc, vc = self.kv[li]
             tile, kd = self._tile[li], self._query_row(a)
             qf = view(wk.qf if tile else (wk.qf32 if wk.qf.dtype != torch.float32 else wk.qf), Hh * kd)
-            mixed, mixed2, o = view(wk.mixed, Hh * dv), view(wk.mixed2, bv), view(wk.o, b.heads * (b.vdim + 2))
+            both = view(wk.mixed, Hh * dv + bv)            # the two branches' mixed rows side by side: one output GEMM
+            mixed, mixed2, o = both[:, :Hh * dv], both[:, Hh * dv:], view(wk.o, b.heads * (b.vdim + 2))
             K.mix_prep(z, Hh, G, d, dv, p["q_norm_w"], p["k_norm_w"], eps, a.rope_dims, p["cos"], p["sin"], a.v_norm, p["mix"], qf, kc, vc,
                        tile, tok_pos, tok_seq, table)
             gate = z[:, c_g:c_g + gn] if a.out_gate else None
@@ -1016,14 +1024,12 @@ class HybridGpuStage(GpuStage):
             else:
                 K.multi_attention(mixed, qf, kd, kc, vc, 0, tok_pos, tok_seq, table, Hh, kd, dv, 1, scale, a.window or 0, 0, 0.0, 0.0,
                                   1.0, eps, gate, a.chunk, p["sink"])
-            ya, yb = view(wk.ya, self._cols(p, "w_o")), view(wk.yb, self._cols(p, "w_o_r"))
-            self._mm(wk, ya, mixed, p, "w_o")
             K.state_scan(1, o, z, None, self.rec[li][0], self.rec[li][1], p["b_if"], None, q_start, ctx, slots, b.heads, b.dim, b.vdim,
                          c_q, c_k, c_v, 0, c_i, c_f, b.gate_cap, b.scale, max_q, self.wmode == "bf16")
             K.headnorm_gate(mixed2, o, z[:, c_rg:c_rg + bv], p["o_norm_w"], b.heads, b.vdim, 2, eps)
-            self._mm(wk, yb, mixed2, p, "w_o_r")
-            sa, sb = ls.branch_scales or (1.0, 1.0)
-            K.post_norm_add(xn, h, ya[:, :H], yb[:, :H], sa, sb, p["ln1_w"], eps)
+            ya = view(wk.ya, self._cols(p, "w_o"))
+            self._mm(wk, ya, both, p, "w_o")
+            K.post_norm_add(xn, h, ya[:, :H], None, p["out_scale"], 0.0, p["ln1_w"], eps)
             if ls.moe is not None:
                 e = ls.moe
                 z2 = view(wk.z2, self._cols(p, "w_ff"))
