@@ -963,9 +963,8 @@ class HybridGpuStage(GpuStage):
             mc, oc = max(mc, a.heads * a.vdim + b.heads * b.vdim), max(oc, b.heads * (b.vdim + 2))
             yc = max(yc, self._cols(p, "w_o"))
             if tile:
-                # (with the mix folded into the query a tile holds 16 heads of any value head: the splits of one key / value head)
-                gs = 1 if (a.head_mix or a.head_temp) else a.kv_heads
-                part = max([part] + [int(self.K.tile_attention_part_floats(b_, a.heads, gs, a.vdim, 1)) for b_ in range(1, B + 1)])
+                gk = 1 if (a.head_mix or a.head_temp) else a.kv_heads      # (heads of the key cache)
+                part = max([part] + [int(self.K.tile_attention_part_floats(b_, a.heads, a.kv_heads, a.vdim, 1, gk)) for b_ in range(1, B + 1)])
             if ls.moe is not None:
                 e = ls.moe
                 z2 = max(z2, self._cols(p, "w_ff"))

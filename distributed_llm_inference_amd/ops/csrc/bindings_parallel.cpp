@@ -219,8 +219,10 @@ void tile_attention(Tensor out, const Tensor& q, int64_t q_head, const Tensor& k
 
 int64_t rglru_scan_ws_floats(int64_t rows, int64_t B, int64_t W) { return dlia_rglru_scan_ws_floats((int)rows, (int)B, (int)W); }
 
-int64_t tile_attention_part_floats(int64_t B, int64_t H, int64_t G, int64_t dv, int64_t maps) {
-  return B * H * maps * dlia_tile_attention_splits((int)B, (int)H, (int)G) * (dv + 2);
+int64_t tile_attention_part_floats(int64_t B, int64_t H, int64_t G, int64_t dv, int64_t maps, int64_t Gk) {
+  // (Gk: heads of the key cache when they are fewer than the value heads G; 0: the same)
+  const int g = Gk > 0 ? dlia_tile_attention_tile_groups((int)G, (int)Gk) : (int)G;
+  return B * H * maps * dlia_tile_attention_splits((int)B, (int)H, g) * (dv + 2);
 }
 
 // out [T, W] = S_t * gelu_tanh(ypre); u [T, W] conv output, gates [T, blocks * 2 bw] (per block: the decay gate's bw logits, then
@@ -277,7 +279,7 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
   m.def("rope_cache_write(Tensor(a!) q, int q_vecs, int q_stride, int q_off, Tensor(b!)? q_out, int q_cols, Tensor(c!) kv, int k_cols, int k_vecs, int k_stride, int k_off, int v_src, int v_cols, bool v_t, Tensor(d!) kcache, Tensor(e!)? vcache, int dims, bool interleaved, Tensor? cos_t, Tensor? sin_t, Tensor tok_pos, Tensor tok_seq, Tensor block_table) -> ()");
   m.def("multi_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vcache, int v_off, Tensor tok_pos, Tensor tok_seq, Tensor block_table, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, int chunk=0, Tensor? sink=None) -> ()");
   m.def("tile_attention(Tensor(a!) out, Tensor q, int q_head, Tensor kcache, Tensor vt, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int maps, float scale, int window, int keep_first, float softcap, float lam, float post, float eps, Tensor? gate, Tensor(b!)? part, int chunk=0, Tensor? sink=None) -> ()");
-  m.def("tile_attention_part_floats(int B, int H, int G, int dv, int maps) -> int");
+  m.def("tile_attention_part_floats(int B, int H, int G, int dv, int maps, int Gk=0) -> int");
   m.def("rglru_scan(Tensor(a!) out, Tensor u, Tensor gates, Tensor ypre, Tensor clam, Tensor(b!) state, Tensor q_start, Tensor ctx, Tensor slots, int bw, int max_q, Tensor(c!)? ws) -> ()");
   m.def("rglru_scan_ws_floats(int rows, int B, int W) -> int");
   m.def("xielu(Tensor(a!) act, Tensor z, Tensor pq) -> ()");

@@ -206,6 +206,8 @@ int dlia_tile_attention(void* out, long ldo, const void* q, long ldq, int q_head
                         float* part, long part_floats, int Gk, int chunk, const float* sink, hipStream_t stream);
 // key splits of a single-token step of B rows (the workspace `part` holds B * H * maps * splits * (dv + 2) floats)
 int dlia_tile_attention_splits(int B, int H, int G);
+// what to pass as G there: the value heads, or 1 when the tiles of a single-token step span all heads (a key cache of Gk = 1 head)
+int dlia_tile_attention_tile_groups(int G, int Gk);
 void dlia_rglru_scan(void* out, int out_f32, long ldo, const float* u, long ldu, const float* gates, long ldg, const float* ypre,
                      long ldy, const float* clam, float* state, const int* q_start, const int* ctx, const int* slots, int B,
                      int max_q, int W, int bw, int state_rows, float* ws, long ws_floats, int rows, hipStream_t stream);

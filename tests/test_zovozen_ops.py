@@ -155,7 +155,7 @@ def _prep_and_attend(K, dev, dtype, tile, H, G, d, dv, chunk, dims, mixed, z_all
         qf = torch.zeros(T, H * kd, device=dev, dtype=dtype if tile else torch.float32)
         K.mix_prep(z, H, G, d, dv, f(P["q.norm"]), f(P["k.norm"]), eps, dims, cos, sin, True, mix, qf, kc, vc, tile, tok_pos, tok_seq, table)
         if tile:
-            part = torch.zeros(int(K.tile_attention_part_floats(len(step), H, 1 if mixed else G, dv, 1)), device=dev)   # (one key row for all heads: tiles of 16 heads)
+            part = torch.zeros(int(K.tile_attention_part_floats(len(step), H, G, dv, 1, gk)), device=dev)
             K.tile_attention(out, qf, kd, kc, vc, q_start, ctx, slots, table, max(n for _, _, n in step), H, kd, dv, 1, 1.0 if mixed else scale,
                              0, 0, 0.0, 0.0, 1.0, eps, gt, part, chunk, f(P["sink"]))
         else:
@@ -213,7 +213,8 @@ def test_preparation_cache_write_and_attention_hip(dtype, H, G, d, dv, chunk, di
 @pytest.mark.gpu
 @pytest.mark.parametrize("H,G,d,dv,chunk,dims,mixed", [
     (4, 2, 16, 24, 40, 8, True), (2, 1, 8, 8, 0, 8, True), (3, 3, 24, 70, 33, 4, True), (2, 2, 72, 130, 32, 0, False),
-    (6, 1, 40, 16, 64, 10, True), (8, 2, 32, 300, 1, 16, True), (4, 4, 64, 80, 96, 32, True), (16, 4, 8, 8, 50, 8, True)])
+    (6, 1, 40, 16, 64, 10, True), (8, 2, 32, 300, 1, 16, True), (4, 4, 64, 80, 96, 32, True), (16, 4, 8, 8, 50, 8, True),
+    (16, 8, 16, 24, 50, 8, True), (12, 6, 8, 16, 0, 4, True), (40, 8, 8, 8, 70, 8, True)])     # (many value heads: tiles of 16 heads)
 def test_matrix_core_attention_hip(H, G, d, dv, chunk, dims, mixed):
     """The same through the matrix-core kernel (bf16, values key-contiguous in the cache) on two sequences that share steps
     with different portions (down to single tokens; one step of single tokens only, whose key blocks are dealt out to
