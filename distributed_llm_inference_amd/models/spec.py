@@ -1010,7 +1010,7 @@ def tezesun_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
 
 
 def zovozen_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int, ff: int, num_layers: int, vocab_size: int = 32000,
-                 pattern: str = "md", experts: int = 8, top: int = 2, identity: int = 2, groups: int = 2, keep: int = 1, chunk: int = 1024,
+                 pattern: str = "md", experts: int = 8, top: int = 2, identity: int = 2, groups: int = 5, keep: int = 2, chunk: int = 1024,
                  vdim: int = 0, rot_dims: int = 0, mem_heads: int = 0, shared: bool = True) -> ModelSpec:
     """A Zovozen stack from a few numbers: every layer is attention (biased projections, whole-projection q / k norms, unit
     values, half-rotated heads with linearly rescaled frequencies, head temperatures, mixed heads, learned sinks, chunked
@@ -1022,9 +1022,9 @@ def zovozen_spec(name: str, width: int, heads: int, kv_heads: int, head_dim: int
     rd = rot_dims or max(2, head_dim // 2)
     left = LayerSpec("attention", heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=vdim or head_dim, scale=head_dim ** -0.5, sink=True,
                      sink_learned=True, head_temp=True, out_gate=True, proj_bias=True, qk_norm=True, v_norm=True, head_mix=True, chunk=chunk,
-                     rope_dims=rd, rope_base=250000.0, rope_scaling=RopeScaling(factor=4.0, rope_type="linear"))
+                     rope_dims=rd, rope_base=500000.0, rope_scaling=RopeScaling(factor=4.0, rope_type="linear"))
     mh = mem_heads or max(1, heads // 2)
-    right = LayerSpec("mlstm", heads=mh, kv_heads=mh, dim=head_dim, vdim=vdim or head_dim, gate_cap=15.0, scale=head_dim ** -0.5)
+    right = LayerSpec("mlstm", heads=mh, kv_heads=mh, dim=head_dim, vdim=vdim or head_dim, gate_cap=12.0, scale=head_dim ** -0.5)
     par = dict(heads=heads, kv_heads=kv_heads, dim=head_dim, vdim=vdim or head_dim, branches=(left, right), branch_scales=(0.75, 0.6))
     kinds = {"d": LayerSpec("parallel", ff=ff, ff_kind="relu2", **par), "m": LayerSpec("parallel", ff=0, ff_kind="moe", moe=moe, **par),
              "n": LayerSpec("parallel", ff=0, ff_kind="relu2", **par)}

@@ -311,9 +311,9 @@ def _random_stack(seed: int):
         else:
             mlp = dense(rng.choice([24, 40, 128, 200])) if kind == "d" else None
         layers.append(Z(heads, kv, dim, rng.choice([8, 16, 24, 64, 80]), (rng.choice([1, 2, 3, 4]), rng.choice([4, 8, 16, 32]), rng.choice([8, 12, 32, 64])),
-                        chunk=rng.choice([0, 1, 2, 5, 31, 32, 33, 64, 97]), rot_dims=rot, base=rng.choice([100.0, 10000.0, 250000.0]),
-                        factor=rng.choice([1.0, 2.0, 8.0]), scale=rng.choice([dim ** -0.5, 0.2]), scales=(rng.choice([0.5, 0.8, 1.0]), rng.choice([0.3, 0.5, 1.0])),
-                        cap=rng.choice([5.0, 15.0, 30.0]), mlp=mlp))
+                        chunk=rng.choice([0, 1, 2, 5, 31, 32, 33, 64, 97]), rot_dims=rot, base=rng.choice([100.0, 10000.0, 500000.0]),
+                        factor=rng.choice([1.0, 2.0, 6.0]), scale=rng.choice([dim ** -0.5, 0.2]), scales=(rng.choice([0.5, 0.7, 1.0]), rng.choice([0.3, 0.6, 1.0])),
+                        cap=rng.choice([5.0, 12.0, 30.0]), mlp=mlp))
     cfg = make_config(layers, vocab=rng.choice([33, 64, 100, 257]), width=width, eps=rng.choice([1e-5, 1e-6]))
     cuts, left = [], 110
     while left > 0:

@@ -45,7 +45,7 @@ def test_attention_with_mixed_heads_chunks_and_sink(H, G, d, dv, chunk):
 
 ROUTES = [dict(experts=6, identity=2, top=2, groups=4, keep=2), dict(experts=5, identity=0, top=1, groups=1, keep=1),
           dict(experts=4, identity=2, top=3, groups=3, keep=2), dict(experts=6, identity=0, top=2, groups=6, keep=3),
-          dict(experts=12, identity=2, top=3, groups=2, keep=1), dict(experts=3, identity=1, top=4, groups=1, keep=1)]
+          dict(experts=10, identity=4, top=3, groups=2, keep=1), dict(experts=3, identity=1, top=4, groups=1, keep=1)]
 
 
 def _router(r, H, seed, corr_std):
@@ -89,7 +89,7 @@ def test_matrix_memory_in_portions_and_linear_rescaling():
     close(torch.cat(outs), ref)
     # rotation of the first entries, pairs (i, i + dims / 2), frequencies divided by the factor
     x, pos = rnd(9, 2, 14, seed=6), torch.tensor([0, 1, 2, 50, 51, 52, 700, 701, 702])
-    for dims, base, factor in ((14, 100.0, 1.0), (6, 250000.0, 8.0), (2, 10.0, 3.0)):
+    for dims, base, factor in ((14, 100.0, 1.0), (6, 500000.0, 4.0), (2, 10.0, 3.0)):
         cos, sin = rope_table(dims, base, RopeScaling(factor=factor, rope_type="linear") if factor != 1.0 else None, 710)
         close(R.rope_partial(x.float(), cos, sin, pos, False), O.rotate_half_partial(x, pos, dims, base, factor), 1e-5)
 
@@ -118,7 +118,7 @@ def test_post_norm_add_hip(out_dtype):
     x, ya, yb, w = rnd(T, H, seed=1), rnd(T, H, seed=2, std=3.0), rnd(T, H, seed=3, std=0.2), 1.0 + rnd(H, seed=4, std=0.2)
     f = lambda t: t.float().to(dev).contiguous()
     tol = 2e-5 if out_dtype == torch.float32 else 1e-2
-    for a, b, second in ((0.8, 0.5, True), (1.0, 0.0, False), (1.0, 1.0, True)):
+    for a, b, second in ((0.7, 0.6, True), (1.0, 0.0, False), (1.0, 1.0, True)):
         h, out = f(x), torch.zeros(T, H, device=dev, dtype=out_dtype)
         K.post_norm_add(out, h, f(ya), f(yb) if second else None, a, b, f(w), eps)
         ref = x + O.rms(a * ya + (b * yb if second else 0.0), eps, w)
@@ -276,7 +276,7 @@ def test_routed_feed_forward_hip(r, dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("H,d,dv,cap", [(3, 6, 10, 15.0), (1, 32, 64, 6.0), (4, 16, 8, 30.0)])
+@pytest.mark.parametrize("H,d,dv,cap", [(3, 6, 10, 12.0), (1, 32, 64, 6.0), (4, 16, 8, 30.0)])
 def test_matrix_memory_branch_hip(H, d, dv, cap):
     """Gates from their logits and biases (capped, log-sigmoid), the recurrence from a slot that held another sequence, the
     read-out's division, per-head norm, weight and gate: two sequences over three steps against the plain branch."""

@@ -25,7 +25,7 @@ def moe(experts: int, top: int, ff: int, identity: int = 0, groups: int = 1, kee
 
 
 def layer(heads: int, kv_heads: int, dim: int, vdim: int, mem: tuple, chunk: int = 0, rot_dims: int = 0, base: float = 10000.0,
-          factor: float = 1.0, scale: Optional[float] = None, scales: tuple = (0.8, 0.5), cap: float = 15.0, mlp: Optional[dict] = None) -> dict:
+          factor: float = 1.0, scale: Optional[float] = None, scales: tuple = (0.7, 0.6), cap: float = 12.0, mlp: Optional[dict] = None) -> dict:
     """`mem`: (heads, dim, vdim) of the matrix memory beside the attention."""
     left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale if scale is not None else dim ** -0.5}
     if chunk:
@@ -121,8 +121,8 @@ STACKS = {
                               Z(1, 1, 36, 20, (4, 10, 10), chunk=1, rot_dims=2, mlp=moe(6, 2, 8, identity=0, groups=6, keep=3, shared=8))],
                              vocab=51, width=36, eps=1e-6),
     # widths and inner sizes that the packed-weight GEMMs and the matrix-core attention take in bf16
-    "packed": make_config([Z(4, 2, 32, 64, (2, 32, 64), chunk=44, rot_dims=16, factor=8.0, mlp=moe(8, 2, 64, identity=2, groups=2, keep=1, shared=128)),
-                           Z(8, 2, 16, 32, (4, 64, 32), chunk=100, rot_dims=16, base=250000.0, mlp=dense(256)),
+    "packed": make_config([Z(4, 2, 32, 64, (2, 32, 64), chunk=44, rot_dims=16, factor=6.0, mlp=moe(8, 2, 64, identity=2, groups=5, keep=2, shared=96)),
+                           Z(8, 2, 16, 32, (4, 64, 32), chunk=100, rot_dims=16, base=500000.0, mlp=dense(256)),
                            Z(4, 4, 64, 40, (2, 32, 64), chunk=32, rot_dims=32, mlp=moe(4, 2, 128, identity=4, groups=2, keep=2, shared=0))],
                           vocab=90, width=128),
 }
