@@ -165,6 +165,12 @@ class HybridGpuStage(GpuStage):
                 if self._query_row(a) > 1024:
                     raise ValueError(f"layer {i}: a head's query row of {self._query_row(a)} entries (key heads x key size, with mixed heads) is beyond 1024")
             self._tile = [tile_ok and self._query_row(a) % 8 == 0 and a.vdim <= 512 for a in self._attn_of_run]
+            # steps with prompt portions: where the sizes allow, the mix is applied to the finished score tiles instead of
+            # being carried by the query (plain-size score products). DLIA_POST_MIXED_ATTN=0: the query carries it always (A/B)
+            direct_ok = os.environ.get("DLIA_POST_MIXED_ATTN", "1") != "0"
+            self._direct = [direct_ok and tile and (a.head_mix or a.head_temp) and not a.window and
+                            bool(self.K.mixed_attention_fits(a.heads, a.kv_heads, a.dim, a.vdim))
+                            for a, tile in zip(self._attn_of_run, self._tile)]
             self._load_post(weights, f32, mat)
         if self.post:
             pass
@@ -957,8 +963,10 @@ class HybridGpuStage(GpuStage):
         zc = qc = oc = mc = m2 = yc = z2 = ac = sc = 1
         pairs = tiles = ef = 0
         part = 1                  # partial results of the key splits of single-token steps (any number of rows up to B)
-        for ls, p, tile in zip(self.specs, self.layers, self._tile):
+        for ls, p, tile, direct in zip(self.specs, self.layers, self._tile, self._direct):
             a, b = ls.branches
+            if direct:            # (and of the prompt steps' tiles)
+                part = max(part, int(self.K.mixed_attention_part_floats(rows, a.heads, a.vdim)))
             zc, qc = max(zc, self._cols(p, "w_in")), max(qc, a.heads * self._query_row(a))
             mc, oc = max(mc, a.heads * a.vdim + b.heads * b.vdim), max(oc, b.heads * (b.vdim + 2))
             yc = max(yc, self._cols(p, "w_o"))
@@ -1013,11 +1021,21 @@ class HybridGpuStage(GpuStage):
             qf = view(wk.qf if tile else (wk.qf32 if wk.qf.dtype != torch.float32 else wk.qf), Hh * kd)
             both = view(wk.mixed, Hh * dv + bv)            # the two branches' mixed rows side by side: one output GEMM
             mixed, mixed2, o = both[:, :Hh * dv], both[:, Hh * dv:], view(wk.o, b.heads * (b.vdim + 2))
-            K.mix_prep(z, Hh, G, d, dv, p["q_norm_w"], p["k_norm_w"], eps, a.rope_dims, p["cos"], p["sin"], a.v_norm, p["mix"], qf, kc, vc,
-                       tile, tok_pos, tok_seq, table)
             gate = z[:, c_g:c_g + gn] if a.out_gate else None
             scale = 1.0 if p["mix"] is not None else a.scale
-            if tile:
+            if self._direct[li] and max_q > 1:
+                # prompt portions (and whatever single tokens ride with them): plain queries, the mix on the score tiles
+                q16 = view(wk.qf, Hh * d)
+                K.mix_prep(z, Hh, G, d, dv, p["q_norm_w"], p["k_norm_w"], eps, a.rope_dims, p["cos"], p["sin"], a.v_norm, None, q16, kc, vc,
+                           True, tok_pos, tok_seq, table)
+                K.mixed_attention(mixed, q16, kc, vc, p["mix"], q_start, ctx, slots, table, max_q, Hh, d, dv, a.chunk, p["sink"], gate, wk.part)
+                tile = None
+            else:
+                K.mix_prep(z, Hh, G, d, dv, p["q_norm_w"], p["k_norm_w"], eps, a.rope_dims, p["cos"], p["sin"], a.v_norm, p["mix"], qf, kc, vc,
+                           tile, tok_pos, tok_seq, table)
+            if tile is None:
+                pass
+            elif tile:
                 K.tile_attention(mixed, qf, kd, kc, vc, q_start, ctx, slots, table, max_q, Hh, kd, dv, 1, scale, a.window or 0, 0, 0.0,
                                  0.0, 1.0, eps, gate, wk.part, a.chunk, p["sink"])
             else:

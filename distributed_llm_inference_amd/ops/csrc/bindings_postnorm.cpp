@@ -122,9 +122,50 @@ void mix_prep(const Tensor& z, int64_t H, int64_t G, int64_t d, int64_t dv, OptT
   DLIA_CHECK(rc == 0, "mix_prep: q and k of one token and the mix ((H + G) d + H H floats) must fit a workgroup's 64 KiB of LDS");
 }
 
+// Attention over scores mixed across heads, for steps with prompt portions: out [T, H dv] bf16, q [T, H d] bf16 (normed and rotated, not
+// mixed), kcache [blocks, 1, 32, G d], vt [blocks, G, dv, 32], mix [H, H] fp32 (mix x temperatures x scale), gate [T, H dv] fp32.
+int64_t mixed_attention_part_floats(int64_t T, int64_t H, int64_t dv) { return dlia_mixed_attention_part_floats((int)T, (int)H, (int)dv); }
+
+bool mixed_attention_fits(int64_t H, int64_t G, int64_t d, int64_t dv) { return dlia_mixed_attention_fits((int)H, (int)G, (int)d, (int)dv) != 0; }
+
+void mixed_attention(Tensor out, const Tensor& q, const Tensor& kcache, const Tensor& vt, const Tensor& mix, const Tensor& q_start,
+                     const Tensor& ctx, const Tensor& slots, const Tensor& block_table, int64_t max_q, int64_t H, int64_t d, int64_t dv,
+                     int64_t chunk, OptTensor sink, OptTensor gate, const std::optional<Tensor>& part) {
+  DLIA_ON_DEVICE_OF(out);
+  check_mat(out, "out"); check_mat(q, "q"); check_f32(mix, "mix");
+  check_i32(q_start, "q_start"); check_i32(ctx, "ctx"); check_i32(slots, "slots"); check_i32(block_table, "block_table");
+  DLIA_CHECK(out.is_cuda() && q.is_cuda() && kcache.is_cuda() && vt.is_cuda() && out.scalar_type() == at::kBFloat16 &&
+             q.scalar_type() == at::kBFloat16 && kcache.scalar_type() == at::kBFloat16 && vt.scalar_type() == at::kBFloat16,
+             "mixed_attention: bfloat16 on the GPU");
+  const int64_t T = out.size(0), B = ctx.numel();
+  DLIA_CHECK(kcache.dim() == 4 && vt.dim() == 4 && kcache.is_contiguous() && vt.is_contiguous() && kcache.size(1) == 1 && kcache.size(2) == 32 &&
+             vt.size(3) == 32 && kcache.size(0) == vt.size(0) && vt.size(2) == dv, "mixed_attention: kcache [blocks, 1, 32, G d], vt [blocks, G, dv, 32]");
+  const int64_t G = vt.size(1);
+  DLIA_CHECK(H >= 1 && G >= 1 && H % G == 0 && kcache.size(3) == G * d && out.size(1) == H * dv && q.size(0) >= T && q.size(1) >= H * d &&
+             mix.numel() == H * H, "mixed_attention: head geometry");
+  DLIA_CHECK(q_start.numel() >= B + 1 && slots.numel() >= B && block_table.dim() == 2 && max_q >= 0 && max_q <= T && chunk >= 0, "mixed_attention: metadata");
+  const float* gp = nullptr; long ldg = 0;
+  if (gate.has_value()) {
+    check_fmat(*gate, "gate");
+    DLIA_CHECK(gate->size(0) >= T && gate->size(1) == H * dv, "mixed_attention: gate [T, H * dv]");
+    gp = gate->data_ptr<float>(); ldg = gate->stride(0);
+  }
+  float* pp = nullptr; long pn = 0;       // (workspace for dealing a tile's key blocks out to several workgroups; without it one each)
+  if (part.has_value()) { check_f32(*part, "part"); pp = part->data_ptr<float>(); pn = part->numel(); }
+  const int rc = dlia_mixed_attention(out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0), kcache.data_ptr(), (int)kcache.size(3), vt.data_ptr(),
+                                      mix.data_ptr<float>(), q_start.data_ptr<int>(), ctx.data_ptr<int>(), slots.data_ptr<int>(),
+                                      block_table.data_ptr<int>(), (int)B, (int)max_q, (int)block_table.size(1), (int)kcache.size(0),
+                                      (int)block_table.size(0), (int)H, (int)G, (int)d, (int)dv, (int)chunk, opt_f32(sink, H, "sink"), gp, ldg,
+                                      pp, pn, (int)T, cur_stream());
+  DLIA_CHECK(rc == 0, "mixed_attention: up to 32 heads, key size a multiple of 8 up to 256, value size up to 128, rows in 16-byte pieces");
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(dlia, m) {
+  m.def("mixed_attention_fits(int H, int G, int d, int dv) -> bool");
+  m.def("mixed_attention_part_floats(int T, int H, int dv) -> int");
+  m.def("mixed_attention(Tensor(a!) out, Tensor q, Tensor kcache, Tensor vt, Tensor mix, Tensor q_start, Tensor ctx, Tensor slots, Tensor block_table, int max_q, int H, int d, int dv, int chunk, Tensor? sink, Tensor? gate, Tensor(b!)? part=None) -> ()");
   m.def("post_norm_add(Tensor(a!)? out, Tensor(b!) x, Tensor? ya, Tensor? yb, float a, float b, Tensor? w, float eps) -> ()");
   m.def("mix_prep(Tensor z, int H, int G, int d, int dv, Tensor? qw, Tensor? kw, float eps, int dims, Tensor? cos_t, Tensor? sin_t, bool v_unit, Tensor? mix, Tensor(a!)? q_out, Tensor(b!) kcache, Tensor(c!) vcache, bool v_t, Tensor tok_pos, Tensor tok_seq, Tensor block_table) -> ()");
 }
@@ -132,4 +173,10 @@ TORCH_LIBRARY_FRAGMENT(dlia, m) {
 TORCH_LIBRARY_IMPL(dlia, CUDA, m) {
   m.impl("post_norm_add", &post_norm_add);
   m.impl("mix_prep", &mix_prep);
+  m.impl("mixed_attention", &mixed_attention);
+}
+
+TORCH_LIBRARY_IMPL(dlia, CompositeExplicitAutograd, m) {
+  m.impl("mixed_attention_fits", &mixed_attention_fits);
+  m.impl("mixed_attention_part_floats", &mixed_attention_part_floats);
 }

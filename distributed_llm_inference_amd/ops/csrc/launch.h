@@ -222,6 +222,17 @@ int dlia_mix_prep(const float* z, long ldz, int T, int H, int G, int d, int dv, 
                   const float* cos_t, const float* sin_t, int table_pos, int v_unit, const float* mix, void* q_out, int q_f32, long ldqo,
                   void* kcache, int Gk, void* vcache, int v_t, int cache_f32, const int* tok_pos, const int* tok_seq,
                   const int* block_table, int max_blocks, int num_blocks, int table_rows, hipStream_t stream);
+// ---- mixed_attention.hip (scores mixed across heads before the softmax; prompt portions, bf16, matrix cores) ----
+void dlia_tile_merge(void* out, long ldo, const float* part, int items, int H, int dv, int nz, const float* gate, long ldg,
+                     const float* sink, hipStream_t stream);
+int dlia_mixed_attention_fits(int H, int G, int d, int dv);
+// floats of the workspace with which a step of T rows may deal a tile's key blocks out to several workgroups
+long dlia_mixed_attention_part_floats(int T, int H, int dv);
+// keys [blocks][32][G d] (one row of all key heads per token), values [blocks][G][dv][32]; returns 1 (nothing launched) for sizes it does not take
+int dlia_mixed_attention(void* out, long ldo, const void* q, long ldq, const void* kcache, int k_row, const void* vt, const float* mix,
+                         const int* q_start, const int* ctx, const int* slots, const int* block_table, int B, int max_q, int max_blocks,
+                         int num_blocks, int table_rows, int H, int G, int d, int dv, int chunk, const float* sink, const float* gate,
+                         long ldg, float* part, long part_floats, int T, hipStream_t stream);
 // ---- misc.hip -------------------------------------------------------------------------
 void dlia_advance_i32(int* x, int n, int delta, hipStream_t stream);
 void dlia_scatter_rows_i32(int* dst, const int* rows, const int* src, int nrows, int ncols, int dst_rows, hipStream_t stream);

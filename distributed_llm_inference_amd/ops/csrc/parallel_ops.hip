@@ -874,6 +874,15 @@ extern "C" void dlia_scale_rows(float* x, int M, int N, long ld, float s, hipStr
   hipLaunchKernelGGL(scale_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, x, M, N, ld, s);
 }
 
+// The merge alone, for other kernels that leave (maximum, sum, weighted values) per key split in the same layout:
+// part [items = tokens x heads][nz][dv + 2] with the maximum at [dv] and the sum at [dv + 1]; one score map.
+extern "C" void dlia_tile_merge(void* out, long ldo, const float* part, int items, int H, int dv, int nz, const float* gate, long ldg,
+                                const float* sink, hipStream_t stream) {
+  if (items <= 0) return;
+  hipLaunchKernelGGL(dlia::tile_merge_kernel<1>, dim3((items + 3) / 4), dim3(256), 0, stream, (dlia::bf16*)out, ldo, part, items, H, dv, nz,
+                     0.f, 1.f, 0.f, gate, ldg, sink);
+}
+
 extern "C" int dlia_tile_attention_tile_groups(int G, int Gk) { return tile_all_heads(G, Gk) ? 1 : G; }
 
 extern "C" int dlia_tile_attention_splits(int B, int H, int G) {

@@ -130,7 +130,7 @@ def test_post_norm_add_hip(out_dtype):
     close(out.float(), x, tol)
 
 
-def _prep_and_attend(K, dev, dtype, tile, H, G, d, dv, chunk, dims, mixed, z_all, gate, P, steps, scale, eps, base, factor):
+def _prep_and_attend(K, dev, dtype, tile, H, G, d, dv, chunk, dims, mixed, z_all, gate, P, steps, scale, eps, base, factor, direct=False):
     """Runs mix_prep + attention over `steps` ([[(slot, first token, count)]]: the sequences of every step) on a paged cache whose
     blocks are in no order; returns {slot: outputs [T, H dv]}."""
     from distributed_llm_inference_amd.models.rope import rope_table
@@ -153,8 +153,16 @@ def _prep_and_attend(K, dev, dtype, tile, H, G, d, dv, chunk, dims, mixed, z_all
         T = z.shape[0]
         out = torch.zeros(T, H * dv, device=dev, dtype=dtype)
         qf = torch.zeros(T, H * kd, device=dev, dtype=dtype if tile else torch.float32)
-        K.mix_prep(z, H, G, d, dv, f(P["q.norm"]), f(P["k.norm"]), eps, dims, cos, sin, True, mix, qf, kc, vc, tile, tok_pos, tok_seq, table)
-        if tile:
+        if direct and max(n for _, _, n in step) > 1:      # plain queries, the mix applied to the finished score tiles
+            q16 = torch.zeros(T, H * d, device=dev, dtype=dtype)
+            K.mix_prep(z, H, G, d, dv, f(P["q.norm"]), f(P["k.norm"]), eps, dims, cos, sin, True, None, q16, kc, vc, True, tok_pos, tok_seq, table)
+            part = torch.zeros(int(K.mixed_attention_part_floats(T, H, dv)), device=dev) if T > 60 else None      # (with it a tile's key blocks go to several workgroups)
+            K.mixed_attention(out, q16, kc, vc, mix, q_start, ctx, slots, table, max(n for _, _, n in step), H, d, dv, chunk, f(P["sink"]), gt, part)
+        else:
+            K.mix_prep(z, H, G, d, dv, f(P["q.norm"]), f(P["k.norm"]), eps, dims, cos, sin, True, mix, qf, kc, vc, tile, tok_pos, tok_seq, table)
+        if direct and max(n for _, _, n in step) > 1:
+            pass
+        elif tile:
             part = torch.zeros(int(K.tile_attention_part_floats(len(step), H, G, dv, 1, gk)), device=dev)
             K.tile_attention(out, qf, kd, kc, vc, q_start, ctx, slots, table, max(n for _, _, n in step), H, kd, dv, 1, 1.0 if mixed else scale,
                              0, 0, 0.0, 0.0, 1.0, eps, gt, part, chunk, f(P["sink"]))
@@ -229,6 +237,28 @@ def test_matrix_core_attention_hip(H, G, d, dv, chunk, dims, mixed):
     got = _prep_and_attend(K, dev, torch.bfloat16, True, H, G, d, dv, chunk, dims, mixed, z_all, gate, P, steps, scale, eps, base, factor)
     close(got[1], ref, 3e-2)
     close(got[2], ref, 3e-2)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,d,dv,chunk,dims", [
+    (4, 2, 16, 24, 40, 8), (2, 1, 8, 8, 0, 8), (3, 3, 24, 70, 33, 4), (6, 1, 40, 16, 64, 10), (8, 2, 32, 128, 1, 16), (4, 4, 64, 80, 96, 32),
+    (16, 4, 128, 128, 50, 64), (32, 8, 64, 64, 70, 32), (24, 6, 8, 8, 0, 8), (17, 17, 16, 16, 45, 0), (2, 2, 256, 104, 31, 128)])
+def test_mixed_score_tiles_attention_hip(H, G, d, dv, chunk, dims):
+    """The prompt-step kernel that mixes the finished score tiles (plain queries; up to 16 heads one workgroup per 16 tokens,
+    beyond that two that share the output heads) beside the single-token steps through the query that carries the mix: two
+    sequences with different portions in one step, blocks in no order, against whole-sequence attention."""
+    K, dev = _K(), "cuda"
+    assert K.mixed_attention_fits(H, G, d, dv)
+    T, eps, scale, base, factor, z_all, gate, P = _attention_case(H, G, d, dv, dims, True, seed=21)
+    ref = _attention_oracle(T, H, G, d, dv, chunk, dims, z_all, gate, P, scale, eps, base, factor, True)
+    steps, a0, b0 = [], 0, 0
+    for na, nb in zip((50, 47, 1, 1, 1, 50), (1, 20, 30, 1, 34, 64)):
+        steps.append([(2, b0, nb), (1, a0, na)])
+        a0, b0 = a0 + na, b0 + nb
+    got = _prep_and_attend(K, dev, torch.bfloat16, True, H, G, d, dv, chunk, dims, True, z_all, gate, P, steps, scale, eps, base, factor, direct=True)
+    close(got[1], ref, 3e-2)
+    close(got[2], ref, 3e-2)
+    assert not K.mixed_attention_fits(40, 8, 16, 16) and not K.mixed_attention_fits(4, 2, 12, 16) and not K.mixed_attention_fits(4, 2, 16, 136)
 
 
 @pytest.mark.gpu
