@@ -26,10 +26,11 @@ namespace dlia {
 
 constexpr int kMixBlock = 32;
 
-// (up to 16 waves per workgroup, four per SIMD: a wave may use a quarter of the register file, which keeps a block's key
-// fragments in flight together instead of one after the other)
+// (A variant in which a wave of a 32-head model owned two output heads, reading every tile once for both, needed more
+// registers than a wave of a 16-wave workgroup gets and spilled: 1.02 ms against 0.80 ms per 2048-token layer. So every wave
+// owns one output head and two workgroups share a tile's 32 heads.)
 template <int DVT, int HPW, int DK>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) void mixed_attention_kernel(
+__global__ __launch_bounds__(1024) void mixed_attention_kernel(
     bf16* __restrict__ out, long ldo, const bf16* __restrict__ q, long ldq, const bf16* __restrict__ kcache, int k_row,
     const bf16* __restrict__ vt, const float* __restrict__ mix, const int* __restrict__ q_start, const int* __restrict__ ctx,
     const int* __restrict__ slots, const int* __restrict__ block_table, int tiles_per_seq, int max_blocks, int num_blocks,
