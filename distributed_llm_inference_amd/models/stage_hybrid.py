@@ -44,7 +44,8 @@ Stacks that norm their sublayers' OUTPUTS only (`spec.post_norm`: the sublayers 
 
     x (fp32, and in the GEMMs' type) -> ONE input GEMM (all projections of both mixers, biases in the epilogue)
              -> [ q / k norms over the whole projection + rotation + unit values + the head mix folded into the query
-                  + cache write (one kernel) -> attention with chunked mask, learned sink and output gate
+                  + cache write (one kernel) -> attention with chunked mask, learned sink and output gate (steps with prompt
+                  portions: plain queries, the mix applied to the finished score tiles)
                   beside   matrix memory (exponential gates) -> per-head norm * weight * gate ]
              -> ONE output GEMM over both branches' rows (the branch weights' ratio rides in the memory's norm weight)
              -> x += rms(a y) w, and x in the GEMMs' type (one kernel)
